@@ -17,7 +17,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ..parts.base import KVBinding, KVCacheNeed, StateBinding, StateNeed
+from ..parts.base import KVBinding, KVCacheNeed, PairBinding, StateBinding, StateNeed
 from .block_manager import GroupSpec
 
 
@@ -42,15 +42,21 @@ def plan_layout(decoder) -> CacheLayout:
         if decoder.cache_owner[i] != i:
             continue
         need = decoder.blocks[layer].mixer.cache_need()
-        if isinstance(need, KVCacheNeed):
-            if need not in needs:
-                needs.append(need)
-            layer_group[i] = needs.index(need)
-        elif isinstance(need, StateNeed):
-            state_layers[i] = need
-        elif need is not None:
-            raise TypeError(f"layer {i}: unknown cache need {need!r}")
-    groups = [GroupSpec(window=n.window, keep_first=n.keep_first) for n in needs] or [GroupSpec()]
+        for one in (need if isinstance(need, tuple) else (need,)):  # (a mixer made of two mixers states a pair of needs)
+            if isinstance(one, KVCacheNeed):
+                if i in layer_group:
+                    raise TypeError(f"layer {i}: one run keeps one set of pages")
+                if one not in needs:
+                    needs.append(one)
+                layer_group[i] = needs.index(one)
+            elif isinstance(one, StateNeed):
+                if i in state_layers:
+                    raise TypeError(f"layer {i}: one run keeps one state")
+                state_layers[i] = one
+            elif one is not None:
+                raise TypeError(f"layer {i}: unknown cache need {one!r}")
+    # (a group with pooled blocks keeps every page: the pooled entries of a request lie in its first pages)
+    groups = [GroupSpec(window=0 if n.pooled_block else n.window, keep_first=0 if n.pooled_block else n.keep_first) for n in needs] or [GroupSpec()]
     return CacheLayout(groups, needs, layer_group, state_layers)
 
 
@@ -62,25 +68,36 @@ class CacheStorage:
         self.spare_slot = num_state_slots
         self.kv: dict[int, tuple[torch.Tensor, torch.Tensor]] = {}
         self.state: dict[int, torch.Tensor] = {}
+        self.pooled: dict[int, tuple[torch.Tensor, torch.Tensor]] = {}
         for i, g in layout.layer_group.items():
             need = layout.group_needs[g]
             k = torch.zeros((num_blocks + 1, need.num_kv_heads, block_size, need.head_dim), dtype=dtype, device=device)
             v = torch.zeros((num_blocks + 1, need.num_kv_heads, need.v_dim, block_size), dtype=dtype, device=device)
             self.kv[i] = (k, v)
+            if need.pooled_block:
+                self.pooled[i] = (torch.zeros_like(k), torch.zeros_like(v))
         for i, need in layout.state_layers.items():
             self.state[i] = torch.zeros((num_state_slots + 1, *need.shape), dtype=need.dtype, device=device)
         for r, owner in enumerate(decoder.cache_owner):
+            pages = state = None
             if owner in self.kv:
                 k, v = self.kv[owner]
-                decoder.bindings[r] = KVBinding(layout.layer_group[owner], k, v, block_size)
-            elif r in self.state:
-                decoder.bindings[r] = StateBinding(self.state[r])
+                kp, vp = self.pooled.get(owner, (None, None))
+                pages = KVBinding(layout.layer_group[owner], k, v, block_size, kp, vp)
+            if r in self.state:
+                state = StateBinding(self.state[r])
+            need = decoder.blocks[decoder.plan.order[r]].mixer.cache_need()
+            if isinstance(need, tuple):  # a mixer made of two mixers: each one's binding, in the order of its needs
+                decoder.bindings[r] = PairBinding(*(pages if isinstance(one, KVCacheNeed) else state if isinstance(one, StateNeed) else None
+                                                    for one in need))
+            elif pages is not None or state is not None:
+                decoder.bindings[r] = pages if pages is not None else state
 
     def kv_bytes_per_token(self) -> int:
         """Bytes of keys and values one token occupies over all runs that own pages."""
         elem = torch.empty((), dtype=self.dtype).element_size()
         return sum(self.layout.group_needs[g].num_kv_heads * (self.layout.group_needs[g].head_dim + self.layout.group_needs[g].v_dim) * elem
-                   for g in self.layout.layer_group.values())
+                   * (2 if self.layout.group_needs[g].pooled_block else 1) for g in self.layout.layer_group.values())
 
     def zero_state(self, slots: list[int]) -> None:
         if self.state and slots:

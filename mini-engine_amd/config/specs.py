@@ -102,6 +102,16 @@ class AttentionSpec:
     query_temperature: tuple[float, int] | None = None
     # a projection to one number per head (role ``g`` of ``names``) whose sigmoid multiplies the head's output
     output_gate: bool = False
+    # "head": q and k are normed head by head (a weight of ``head_dim``); "projection": over all rows of the projection at once,
+    # before they are split into heads (weights of ``num_heads * head_dim`` and ``num_kv_heads * head_dim``)
+    qk_norm_over: str = "head"
+    # the values are the keys as projected, before the norm: there is no value projection (``value_dim`` is ``head_dim``)
+    values_from_keys: bool = False
+    # with a window: beside the window's keys a query sees one key and value for every block of ``pooled_block`` positions that
+    # lies wholly before the window (block b: b P .. b P + P - 1, seen by position i when b P + P - 1 <= i - window): the mean of
+    # the block's keys as the cache holds them and the mean of its values; tokens and blocks share one softmax. Tokens that have
+    # left the window and whose block is not yet complete behind it are not seen
+    pooled_block: int = 0
 
     @property
     def v_dim(self) -> int:
@@ -110,7 +120,9 @@ class AttentionSpec:
     @property
     def kv_elements_per_token(self) -> int:
         """Key and value elements one token occupies in this layer's own pages (none when it reads another's)."""
-        return 0 if self.cache_from is not None else self.num_kv_heads * (self.head_dim + self.v_dim)
+        if self.cache_from is not None:
+            return 0
+        return self.num_kv_heads * (self.head_dim + self.v_dim) * (2 if self.pooled_block else 1)  # (the pooled blocks' pages)
 
 
 @dataclass(frozen=True)
@@ -178,6 +190,50 @@ class DecayStateSpec:
 
 
 @dataclass(frozen=True)
+class DeltaRuleSpec:
+    """Linear attention by the generalized delta rule, with a matrix of state per request and head (``head_dim x head_dim``,
+    float32, zero at first). With r, k, v of ``num_heads x head_dim`` and the unit key ``u = k / sqrt(sum(k^2) + 1e-6)``::
+
+        S_t = diag(w_t) S_(t-1) - (a_t * u_t) (u_t^T S_(t-1)) + k_t v_t^T,     o_t = S_t^T r_t
+
+    (both terms read the old state). The decay per head and key channel is ``w = exp(-decay_coef * sigmoid(W_2 tanh(W_1 h) +
+    w_0))`` with an inner size of ``decay_rank``; the removal rate ``a = sigmoid(W_a h + b_a)``. Each head's output is divided
+    by its root mean square (``norm_eps``); the heads together are multiplied by a weight and by the sigmoid of a gate
+    projection, and go through the output projection. ``names`` maps the roles ``r k v g a a_bias w1 w2 w0 norm o``."""
+
+    hidden_size: int
+    num_heads: int
+    head_dim: int
+    decay_rank: int
+    norm_eps: float
+    decay_coef: float = 0.6065306597126334  # exp(-1/2)
+    names: tuple[tuple[str, str], ...] = ()
+    kind: str = "delta_rule"
+
+    @property
+    def state_elements(self) -> int:
+        return self.num_heads * self.head_dim * self.head_dim
+
+
+@dataclass(frozen=True)
+class PairMixerSpec:
+    """Two mixers side by side that read the same input; the result is ``left_scale * left + right_scale * right``. Their tensors
+    lie under ``<prefix>.<left_name>`` and ``<prefix>.<right_name>``; each keeps a cache or state of its own."""
+
+    left: Any
+    right: Any
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    left_name: str = "left"
+    right_name: str = "right"
+    kind: str = "pair"
+
+    @property
+    def kv_elements_per_token(self) -> int:
+        return sum(int(getattr(m, "kv_elements_per_token", 0)) for m in (self.left, self.right))
+
+
+@dataclass(frozen=True)
 class GatedMlpSpec:
     """Dense gated feed-forward: ``down(act(gate(x)) * up(x))`` without biases; ``activation`` is "silu" or
     "gelu_tanh"."""
@@ -202,6 +258,21 @@ class RoutedExpertsSpec:
     activation: str = "silu"
     names: tuple[tuple[str, str], ...] = ()
     kind: str = "routed_experts"
+    # what an activation with a limit clamps by ("clamped_sigmoid": g = min(gate, limit), u = clamp(up, -limit, limit),
+    # g sigmoid(1.702 g) (u + 1))
+    activation_limit: float = 0.0
+    # "softmax_picked": the picks' weights are the softmax over the picked logits. "sigmoid_normalized": scores are sigmoid(z), the
+    # picks are the largest scores among the experts of the ``keep_groups`` best of ``num_groups`` equal groups of neighbours (a
+    # group's score: the sum of its two largest scores), and the weights are the picks' scores over their sum (+ 1e-20), times
+    # ``route_scale``
+    scoring: str = "softmax_picked"
+    num_groups: int = 1
+    keep_groups: int = 1
+    route_scale: float = 1.0
+    # > 0: one more expert of this size (``<prefix>.<shared>.<gate|up|down>``, the same form, ``shared_limit``) that every token
+    # uses, multiplied by the sigmoid of one number per token (``<prefix>.<shared>.<shared_gate>`` ``[1, hidden]``)
+    shared_size: int = 0
+    shared_limit: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -220,7 +291,8 @@ class LayerSpec:
 
     ``arrangement == "pre_norm"``: ``x += mixer(norm1(x)); x += ffn(norm2(x))``.
     ``arrangement == "parallel"``: ``h = norm1(x); x += residual_scale * (mixer(h) + ffn(h))``: one norm (``mixer_norm``)
-    that both parts read; ``ffn`` may be None (then ``ffn_norm`` and its names are not used).
+    that both parts read; ``ffn`` may be None (then ``ffn_norm`` and its names are not used). With an ``ffn_norm`` the
+    feed-forward has a norm of its own, of the same x: ``x += residual_scale * (mixer(norm1(x)) + ffn(norm2(x)))``.
     ``arrangement == "hyper_connections"``: as ``pre_norm`` over several residual streams: each part reads and rewrites them by
     its :class:`HyperConnectionSpec` (``mixer_streams``, ``ffn_streams``); ``ffn`` may be None.
     The ``*_prefix`` / ``*_name`` strings are the checkpoint names of this layer's tensors.

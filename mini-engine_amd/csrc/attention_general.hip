@@ -47,7 +47,8 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
     const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table,
     int table_width, T* __restrict__ out, int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
     const float* __restrict__ unturn, int un_pairing, float scale, int wpu, const float* __restrict__ sink,
-    const T* __restrict__ gate, size_t gate_row) {
+    const T* __restrict__ gate, size_t gate_row, const T* __restrict__ k_pool, const T* __restrict__ v_pool, int pool,
+    long long out_row, int out_col, float out_scale) {
   constexpr int DMAX = KMAX * ME_WAVE;  // the largest head this instance takes
   __shared__ float qs[8][DMAX];
   __shared__ float parts[8][DMAX + 2];  // with several waves per unit: a round's results (values, maximum, sum)
@@ -61,6 +62,9 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
   int lo = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
   int kept = keep_first < lo ? keep_first : lo;  // keys 0 .. kept-1 are visible beside lo .. p
   if (kept == lo) lo = 0, kept = 0;              // the two runs meet: one run from 0
+  // Pooled blocks: entry b of the pooled pages stands for the positions b pool .. b pool + pool - 1 and is visible once the
+  // window has passed all of them. The entries 0 .. kept-1 are a run of their own, walked like kept first keys.
+  if (pool > 0) kept = lo / pool;
   const int kept_chunks = (kept + AG_CHUNK - 1) / AG_CHUNK;
   const int* table = block_table + (size_t)token_item[t] * table_width;
 
@@ -92,9 +96,11 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
       const int key = tile + lane;
       const bool valid = key >= vlo && key <= vhi;
       float s = -INFINITY;
+      const T* kc = of_kept && pool > 0 ? k_pool : k_cache;
+      const T* vc = of_kept && pool > 0 ? v_pool : v_cache;
       if (valid) {
         const int page = table[key / bs];
-        const T* krow = k_cache + (((size_t)page * nkv + kvh) * bs + key % bs) * d;
+        const T* krow = kc + (((size_t)page * nkv + kvh) * bs + key % bs) * d;
         float dot = 0.f;
         if (vec_k) {  // the same products in the same order; 128 elements of the row are requested before the first is used
           const float4* k4 = reinterpret_cast<const float4*>(krow);
@@ -134,7 +140,7 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
         for (; j <= j_hi && (j & 3); ++j) {
           const float pj = __shfl(pr, j, ME_WAVE);
           const int kj = tile + j;
-          const T* vbase = v_cache + ((size_t)table[kj / bs] * nkv + kvh) * dv * bs + kj % bs;
+          const T* vbase = vc + ((size_t)table[kj / bs] * nkv + kvh) * dv * bs + kj % bs;
 #pragma unroll
           for (int k = 0; k < KMAX; ++k) {
             const int i = lane + k * ME_WAVE;
@@ -149,7 +155,7 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
           for (int gq = 0; gq < 8; ++gq) {
             const bool there = g0 + gq < groups;
             const int kj = tile + j + 4 * (there ? g0 + gq : 0);
-            const T* vbase = v_cache + ((size_t)table[kj / bs] * nkv + kvh) * dv * bs + kj % bs;
+            const T* vbase = vc + ((size_t)table[kj / bs] * nkv + kvh) * dv * bs + kj % bs;
 #pragma unroll
             for (int k = 0; k < KMAX; ++k) {
               const int i = lane + k * ME_WAVE;
@@ -181,7 +187,7 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
         const float pj = __shfl(pr, j, ME_WAVE);
         const int kj = tile + j;
         const int page = table[kj / bs];
-        const T* vbase = v_cache + ((size_t)page * nkv + kvh) * dv * bs + kj % bs;
+        const T* vbase = vc + ((size_t)page * nkv + kvh) * dv * bs + kj % bs;
 #pragma unroll
         for (int k = 0; k < KMAX; ++k) {
           const int i = lane + k * ME_WAVE;
@@ -209,14 +215,14 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
     }
   }
   if (w != 0) return;
-  T* orow = out + ((size_t)t * nh + head) * dv;
+  T* orow = out + (size_t)t * out_row + out_col + (size_t)head * dv;
   if (sink) {  // one more term exp(sink) in the denominator, with no value: a chunk of its own, merged last
     float none[KMAX];
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) none[k] = 0.f;
     ag_merge<KMAX>(mt, lt, acct, sink[head], 1.f, none);
   }
-  float inv = 1.f / lt;
+  float inv = out_scale / lt;
   if (gate) inv *= 1.f / (1.f + expf(-to_float(gate[(size_t)t * gate_row + head])));  // the head's output gate
   if (unturn) {  // the sum of turned values, turned back by this token's angles: through this wave's row of LDS
     __builtin_amdgcn_wave_barrier();
@@ -459,19 +465,29 @@ __global__ __launch_bounds__(1024) void attention_shared_f32_kernel(
 // sink (float32 [nh] or null): a learned logit per head that counts once in the softmax's denominator and has no value (it
 // is not multiplied by the scale). gate (or null; gate[t * gate_row + head] in the activations' type): every head's output
 // is multiplied by the sigmoid of its gate before it is rounded.
-extern "C" int me_attention_general_gated(const void* q, const void* k_cache, const void* v_cache, const int* positions,
-                                          const int* token_item, const int* block_table, int table_width, void* out,
-                                          int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
-                                          const float* unturn, int un_pairing, float scale, const float* sink, const void* gate,
-                                          long long gate_row, int dtype, int items, hipStream_t stream) {
+// k_pool, v_pool, pool: pages of pooled blocks (entry b at page table[b / bs], slot b % bs: the mean of the keys and of the
+// values at the positions b pool .. b pool + pool - 1) that are visible, beside the window's keys, once the window has passed
+// them wholly; they share the softmax with the window's keys. out_row, out_col: the result's rows are out_row elements apart
+// (0: nh * dv) and begin at column out_col; out_scale multiplies the result before it is rounded.
+extern "C" int me_attention_general_pooled(const void* q, const void* k_cache, const void* v_cache, const int* positions,
+                                           const int* token_item, const int* block_table, int table_width, void* out,
+                                           int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
+                                           const float* unturn, int un_pairing, float scale, const float* sink, const void* gate,
+                                           long long gate_row, const void* k_pool, const void* v_pool, int pool, long long out_row,
+                                           int out_col, float out_scale, int dtype, int items, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
+  if (pool < 0 || (pool > 0 && (window <= 0 || keep_first > 0 || !k_pool || !v_pool)))
+    return me_fail("me_attention_general: pooled blocks of %d keys need a window, pages of their own and no kept first keys", pool);
+  if (out_col < 0 || (out_row > 0 && out_col + (long long)nh * dv > out_row))
+    return me_fail("me_attention_general: the result at column %d of a row of %lld", out_col, out_row);
   if (d <= 0 || d > AG_MAX_D_WIDE) return me_fail("me_attention_general: head_dim=%d must be in 1..%d", d, AG_MAX_D_WIDE);
   if (dv <= 0 || dv > AG_MAX_D_WIDE) return me_fail("me_attention_general: value head size %d must be in 1..%d", dv, AG_MAX_D_WIDE);
   const bool big = d > AG_MAX_D || dv > AG_MAX_D;  // the instance with eight elements a lane
   if (keep_first < 0 || (keep_first > 0 && window <= 0))
     return me_fail("me_attention_general: keep_first=%d needs a window", keep_first);
   if (unturn && (dv % 2 || (un_pairing & ~1))) return me_fail("me_attention_general: values of size %d, pairing %d", dv, un_pairing);
-  const bool plain = dv == d && keep_first == 0 && !unturn && !sink && !gate && !big;
+  const bool plain = dv == d && keep_first == 0 && !unturn && !sink && !gate && !big && pool == 0 && out_row <= 0 && out_col == 0 &&
+                     out_scale == 1.f;
   if (nh <= 0 || nkv <= 0 || nh % nkv)
     return me_fail("me_attention_general: %d query heads are not a multiple of %d key/value heads", nh, nkv);
   if (bs <= 0 || table_width <= 0 || window < 0)
@@ -516,7 +532,8 @@ extern "C" int me_attention_general_gated(const void* q, const void* k_cache, co
 #define ME_AG_LAUNCH(TT, KK)                                                                                                   \
   attention_general_kernel<TT, KK><<<blocks, waves * 64, 0, stream>>>(                                                         \
       (const TT*)q, (const TT*)k_cache, (const TT*)v_cache, positions, token_item, block_table, table_width, (TT*)out, num_tokens, \
-      nh, nkv, d, dv, bs, window, keep_first, unturn, un_pairing, scale, wpu, sink, (const TT*)gate, (size_t)gate_row)
+      nh, nkv, d, dv, bs, window, keep_first, unturn, un_pairing, scale, wpu, sink, (const TT*)gate, (size_t)gate_row,             \
+      (const TT*)k_pool, (const TT*)v_pool, pool, out_row > 0 ? out_row : (long long)nh * dv, out_col, out_scale)
   if (dtype == ME_F32) {
     if (big)
       ME_AG_LAUNCH(float, AG_MAX_D_WIDE / ME_WAVE);
@@ -530,6 +547,16 @@ extern "C" int me_attention_general_gated(const void* q, const void* k_cache, co
   }
 #undef ME_AG_LAUNCH
   return me_check_launch("me_attention_general");
+}
+
+extern "C" int me_attention_general_gated(const void* q, const void* k_cache, const void* v_cache, const int* positions,
+                                          const int* token_item, const int* block_table, int table_width, void* out,
+                                          int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
+                                          const float* unturn, int un_pairing, float scale, const float* sink, const void* gate,
+                                          long long gate_row, int dtype, int items, hipStream_t stream) {
+  return me_attention_general_pooled(q, k_cache, v_cache, positions, token_item, block_table, table_width, out, num_tokens, nh, nkv,
+                                     d, dv, bs, window, keep_first, unturn, un_pairing, scale, sink, gate, gate_row, nullptr, nullptr,
+                                     0, 0, 0, 1.f, dtype, items, stream);
 }
 
 extern "C" int me_attention_general_ext(const void* q, const void* k_cache, const void* v_cache, const int* positions,

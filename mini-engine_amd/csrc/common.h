@@ -60,7 +60,9 @@ __device__ __forceinline__ me_u32x2 stream_load8(const void* p) {
 
 // ------------------------------------------------------------------ the activation of a gated feed-forward
 // act(gate) * up: the codes that the entry points' `gated` arguments take (0: the product is not gated).
-enum MeGate { ME_GATE_NONE = 0, ME_GATE_SILU = 1, ME_GATE_GELU_TANH = 2 };
+// ME_GATE_CLAMPED_SIGMOID (kernels that take a limit beside the code): g' = min(gate, limit), u' = clamp(up, -limit, limit),
+// g' sigmoid(1.702 g') (u' + 1).
+enum MeGate { ME_GATE_NONE = 0, ME_GATE_SILU = 1, ME_GATE_GELU_TANH = 2, ME_GATE_CLAMPED_SIGMOID = 3 };
 
 __device__ __forceinline__ float gate_act(float g, int code) {
   if (code == ME_GATE_GELU_TANH) {  // 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
@@ -68,6 +70,15 @@ __device__ __forceinline__ float gate_act(float g, int code) {
     return 0.5f * g * (1.f + tanhf(u));
   }
   return g / (1.f + expf(-g));  // silu
+}
+// act(gate) * up for every code, the forms with a limit among them.
+__device__ __forceinline__ float gated_pair(float g, float u, int code, float limit) {
+  if (code == ME_GATE_CLAMPED_SIGMOID) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+  }
+  return gate_act(g, code) * u;
 }
 // The same for results that are rounded to bfloat16: the exponential and the reciprocal as one instruction each (a
 // correctly rounded division and expf are two dozen instructions at the tail of every gated product).

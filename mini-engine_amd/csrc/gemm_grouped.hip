@@ -28,7 +28,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_grouped_kernel(const bf16_t
                                                                      const int* __restrict__ plan, const int* __restrict__ sorted,
                                                                      const float* __restrict__ wts, bf16_t* __restrict__ acts,
                                                                      float* __restrict__ parts, int num_tokens, int N, int K,
-                                                                     int top, int n_tiles, int gate) {
+                                                                     int top, int n_tiles, int gate, float limit) {
   constexpr int THREADS = WM * WN * 64;
   constexpr int WMR = BM / WM, WNR = BN / WN;
   constexpr int FM = WMR / 16, FN = WNR / 16;
@@ -122,7 +122,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_grouped_kernel(const bf16_t
         const int n = n0 + wn * (WNR / 2) + a * 16 + 4 * g;
         float v[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = gate_act_bf16(acc[a][b][i], gate) * acc[a + FN / 2][b][i];
+        for (int i = 0; i < 4; ++i)
+          v[i] = gate == ME_GATE_CLAMPED_SIGMOID ? gated_pair(acc[a][b][i], acc[a + FN / 2][b][i], gate, limit)
+                                                 : gate_act_bf16(acc[a][b][i], gate) * acc[a + FN / 2][b][i];
         bf16_t* p = acts + (size_t)(begin + m) * N + n;
         if (n + 3 < N && (((uintptr_t)p) & 7) == 0) {
           const gg_bf16x4 w = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
@@ -154,7 +156,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_grouped_kernel(const bf16_t
 
 template <bool GATED>
 int launch_grouped(const bf16_t* X, const bf16_t* W, const int* plan, const int* sorted, const float* wts, bf16_t* acts, float* parts,
-                   int num_tokens, int N, int K, int top, int max_tiles, int gate, hipStream_t stream) {
+                   int num_tokens, int N, int K, int top, int max_tiles, int gate, float limit, hipStream_t stream) {
   constexpr int BM = 128, BN = 128, WM = 4, WN = 2;
   constexpr int COLS = GATED ? BN / 2 : BN;
   constexpr size_t LDS = (size_t)2 * (BM + BN) * GGK * sizeof(bf16_t);
@@ -168,7 +170,7 @@ int launch_grouped(const bf16_t* X, const bf16_t* W, const int* plan, const int*
   const int n_tiles = (N + COLS - 1) / COLS;
   if ((long long)max_tiles * n_tiles > 0x7fffffffLL) return me_fail("me_gemm_grouped: %d x %d blocks exceed the grid", max_tiles, n_tiles);
   hipLaunchKernelGGL(kernel, dim3((unsigned)(max_tiles * n_tiles)), dim3(WM * WN * 64), LDS, stream, X, W, plan, sorted, wts, acts, parts,
-                     num_tokens, N, K, top, n_tiles, gate);
+                     num_tokens, N, K, top, n_tiles, gate, limit);
   return me_check_launch("me_gemm_grouped");
 }
 }  // namespace
@@ -177,15 +179,17 @@ int launch_grouped(const bf16_t* X, const bf16_t* W, const int* plan, const int*
 extern "C" int me_gemm_grouped_tile_rows() { return 128; }
 
 // gated != 0: acts [P, N] = act(x_e . Wg_e^T) * (x_e . Wu_e^T), x rows gathered by token (W [E, 2 N, K]); else
+// (limit: what the activations with a limit clamp by)
 // parts [top, tokens, N] = weight * (acts_e . Wd_e^T) (W [E, N, K], X = acts [P, K]). max_tiles: an upper bound of the list's length.
 extern "C" int me_gemm_grouped_bf16(const void* X, const void* W, const int* plan, const int* sorted, const float* wts, void* acts,
-                                    float* parts, int num_tokens, int N, int K, int top, int max_tiles, int gated, hipStream_t stream) {
+                                    float* parts, int num_tokens, int N, int K, int top, int max_tiles, int gated, float limit,
+                                    hipStream_t stream) {
   if (num_tokens <= 0 || max_tiles <= 0) return 0;
   if (K <= 0 || K % GGK) return me_fail("me_gemm_grouped: K=%d must be a positive multiple of %d", K, GGK);
   if (((uintptr_t)X | (uintptr_t)W) & 15) return me_fail("me_gemm_grouped: operands must be 16-byte aligned");
   if (gated)
     return launch_grouped<true>((const bf16_t*)X, (const bf16_t*)W, plan, sorted, wts, (bf16_t*)acts, nullptr, num_tokens, N, K, top,
-                                max_tiles, gated, stream);
+                                max_tiles, gated, limit, stream);
   return launch_grouped<false>((const bf16_t*)X, (const bf16_t*)W, plan, sorted, wts, nullptr, parts, num_tokens, N, K, top, max_tiles, 0,
-                               stream);
+                               0.f, stream);
 }

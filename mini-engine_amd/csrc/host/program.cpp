@@ -219,7 +219,19 @@ class Run {
         norm_linear(op);
         break;
       case kOpNorm:
+        if (op.i[1]) {  // a second norm of the same stream: nothing is added, what was set aside stays aside
+          if (pending_.any() || pending_.carried()) throw Error(kBroken, "a result is pending before a second norm of the stream");
+          ok(me_add_group_rmsnorm2(x_, nullptr, nullptr, 0, 0, nullptr, nullptr, 0, 0, 1.f, (const float*)op.p[0], bufs_[op.out], nullptr,
+                                   t_, h_, groups_of(op.i[0]), op.f[0], 0, dtype_, stream_));
+          break;
+        }
         add_norm((const float*)op.p[0], op.f[0], bufs_[op.out], groups_of(op.i[0]));
+        break;
+      case kOpPooledAttention:
+        pooled_attention(op);
+        break;
+      case kOpDeltaRule:
+        delta_rule(op);
         break;
       case kOpLinear:
         product(bufs_[op.in], op.p[1], (int)op.i[0], (int)op.i[1], (int)op.i[2], dtype_, bufs_[op.out]);
@@ -757,19 +769,57 @@ class Run {
                        t_, nh, dv, rank, dtype_, stream_));
   }
 
-  // A feed-forward of routed experts (csrc/routed_ff.hip): its result waits as one partial sum per expert of a token.
+  // A feed-forward of routed experts (csrc/routed_ff.hip): its result waits as one partial sum per expert of a token, and one
+  // more for an expert that every token uses (two plain products around the activation, which the token's gate multiplies).
   void routed_ff(const Op& op) {
-    const int E = (int)op.i[0], top = (int)op.i[1], ff = (int)op.i[2];
+    const int E = (int)op.i[0], top = (int)op.i[1], ff = (int)op.i[2], shared_ff = (int)op.i[7];
     pending_ = Pending();
+    pending_.scale = scale_of(op.f[3]);  // what the block multiplies the result by
     parts_mark_ = arena_.used;
-    float* parts = (float*)arena_.take((size_t)top * t_ * h_ * 4);
+    const int sums = top + (shared_ff > 0 ? 1 : 0);
+    float* parts = (float*)arena_.take((size_t)sums * t_ * h_ * 4);
     released_to_ = arena_.used;  // the partial sums outlive this operation, its workspace does not
     void* ws = arena_.take((size_t)me_routed_ff_workspace(t_, E, top, ff, elem_));
-    ok(me_routed_ff(bufs_[op.in], (const float*)op.p[0], op.p[1], op.p[2], parts, ws, t_, h_, E, top, ff, (int)op.i[3], dtype_,
-                    stream_));
+    float* shared_gate = shared_ff > 0 ? (float*)arena_.take((size_t)t_ * 4) : nullptr;
+    ok(me_routed_ff_scored(bufs_[op.in], (const float*)op.p[0], op.p[1], op.p[2], parts, ws, t_, h_, E, top, ff, (int)op.i[3], op.f[0],
+                           (int)op.i[4], (int)std::max<int64_t>(op.i[5], 1), (int)std::max<int64_t>(op.i[6], 1), scale_of(op.f[1]),
+                           shared_gate, dtype_, stream_));
+    if (shared_ff > 0) {
+      void* gu = arena_.take((size_t)t_ * 2 * shared_ff * elem_);
+      void* act = arena_.take((size_t)t_ * shared_ff * elem_);
+      product(bufs_[op.in], op.p[3], 2 * shared_ff, h_, 0, dtype_, gu);
+      ok(me_gated_rows(gu, shared_gate, act, t_, shared_ff, (int)op.i[3], op.f[2], dtype_, stream_));
+      product(act, op.p[4], h_, shared_ff, 0, kF32, parts + (size_t)top * t_ * h_);
+    }
     pending_.parts = parts;
-    pending_.num_parts = top;
+    pending_.num_parts = sums;
     pending_.stride = (long long)t_ * h_;
+  }
+
+  // Attention over a sliding window and the means of whole blocks of keys before it (csrc/pooled_attention.hip, then the general
+  // attention kernel with the pooled entries as a run of their own).
+  void pooled_attention(const Op& op) {
+    const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2], dv = (int)op.i[3], bs = (int)op.i[4];
+    const int window = (int)op.i[5], pool = (int)op.i[6], g = (int)op.i[7];
+    if (g < 0 || g >= (int)s_.lay.widths.size()) throw Error(kBadValue, "an attention layer names a cache group the step lacks");
+    const int32_t* table = idx(s_.lay.tables[g]);
+    const int width = s_.lay.widths[g];
+    const long long row = values_[op.in].cols, out_row = values_[op.out].cols;
+    void* q = arena_.take((size_t)t_ * nh * d * elem_);
+    ok(me_whole_norm_scatter(bufs_[op.in], row, (int)op.i[8], (int)op.i[9], (int)op.i[10], (const float*)op.p[0], (const float*)op.p[1],
+                             idx(s_.lay.positions), idx(s_.lay.token_item), table, width, q, (void*)op.p[2], (void*)op.p[3],
+                             (void*)op.p[4], (void*)op.p[5], t_, nh, nkv, d, dv, bs, pool, op.f[0], dtype_, stream_));
+    ok(me_attention_general_pooled(q, op.p[2], op.p[3], idx(s_.lay.positions), idx(s_.lay.token_item), table, width, bufs_[op.out], t_, nh,
+                                   nkv, d, dv, bs, window, 0, nullptr, 0, op.f[1], nullptr, nullptr, 0, op.p[4], op.p[5], pool, out_row,
+                                   (int)op.i[11], scale_of(op.f[2]), dtype_, s_.lay.items, stream_));
+  }
+
+  // Linear attention by the generalized delta rule over the state rows of the step's items (csrc/delta_rule.hip).
+  void delta_rule(const Op& op) {
+    ok(me_delta_rule(bufs_[op.in], values_[op.in].cols, (int)op.i[3], (int)op.i[4], (int)op.i[5], (int)op.i[6], (int)op.i[7], (int)op.i[8],
+                     op.p[0], (const float*)op.p[1], (const float*)op.p[2], (const float*)op.p[3], (float*)op.p[4],
+                     idx(s_.lay.item_start), idx(s_.lay.state_slots), bufs_[op.out], values_[op.out].cols, (int)op.i[9],
+                     scale_of(op.f[2]), t_, s_.lay.items, (int)op.i[0], (int)op.i[1], (int)op.i[2], op.f[0], op.f[1], dtype_, stream_));
   }
 
   // Rows are selected before the final norm, as the reference does (model.py:186); logits are float32.
@@ -916,8 +966,9 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
       }
     }
     if (op.kind == kOpRoutedFF)
-      need = (size_t)op.i[1] * tokens * hidden_ * 4 + (size_t)me_routed_ff_workspace(tokens, (int)op.i[0], (int)op.i[1], (int)op.i[2], (int)elem) +
-             2 * pad;
+      need = (size_t)(op.i[1] + 1) * tokens * hidden_ * 4 + (size_t)me_routed_ff_workspace(tokens, (int)op.i[0], (int)op.i[1], (int)op.i[2], (int)elem) +
+             (size_t)tokens * (4 + 3 * op.i[7] * elem + 2 * op.i[7] * 4) + 6 * pad;
+    if (op.kind == kOpPooledAttention) need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;
     if (op.kind == kOpAttention && !attention_is_plain(op)) {
       need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;
       if (attention_takes_tiled_prefill(op, dtype_)) {  // the splits' partial results of a decode step

@@ -26,7 +26,8 @@ enum OpKind {
   kOpEmbed = 0,       // p0 table, f0 the multiplier on the looked-up rows; -> x
   kOpNormLinear = 1,  // p0 norm weight, f0 eps, p1 W [rows, K], i0 rows of W, i1 K, i2 gated, i3 groups of the norm (0: one);
                       // pending + x -> out
-  kOpNorm = 2,        // p0 norm weight, f0 eps, i0 groups of the norm (0: one); pending + x -> out [tokens, hidden]
+  kOpNorm = 2,        // p0 norm weight, f0 eps, i0 groups of the norm (0: one); pending + x -> out [tokens, hidden]. i1 != 0: a second
+                      // norm of the same stream (nothing is pending; a result that was set aside stays aside)
   kOpLinear = 3,      // in, p1 W, i0 rows of W, i1 K, i2 gated -> out
   kOpLinearDelta = 4, // in, p1 W, i0 rows of W (= hidden), i1 K, f0 what the block multiplies the delta by (0: 1) -> pending
   kOpDelta = 5,       // in, f0 what the block multiplies the delta by (0: 1) -> pending
@@ -65,10 +66,23 @@ enum OpKind {
                       // f0 eps, f1 scale -> out [tokens, heads * dv]
   kOpRoutedFF = 18,   // in: normed activations; p0 router W float32 [E, hidden], p1 experts' gate and up rows [E, 2 ff, hidden],
                       // p2 experts' down rows [E, hidden, ff]; i0 E, i1 experts a token, i2 ff, i3 code of the activation
-                      // -> pending (partial sums, one per expert of a token)
+                      // -> pending (partial sums, one per expert of a token). f0 the activation's limit; i4 how the picks are scored
+                      // (0: softmax over the picked logits; 1: sigmoid scores over their sum, times f1, picks bounded to the i6 best of
+                      // i5 groups). i7 > 0: an expert of that size that every token uses, p3 its gate and up rows [2 i7, hidden], p4
+                      // its down rows [hidden, i7], f2 its limit; the router then has one more row, whose sigmoid multiplies it. f3 what the block
+                      // multiplies the result by (0: 1)
   kOpStreamNormLinear = 19,  // kOpStreamNorm and the product behind it: p0 norm weight, f0 eps, p1 W [rows, hidden], p2 how the pending
                       // result rewrites the streams (or null), p3 what the product's part reads of each stream; i0 rows of W, i1 K,
                       // i2 gated; pending + streams -> streams, out
+  kOpPooledAttention = 20,  // attention over a window and the means of whole blocks of keys before it. in: projections, queries at column
+                      // i8 (heads * d), keys at i9 (kv heads * d), values at i10 (kv heads * dv; -1: the values are the keys as projected);
+                      // p0, p1 float32 weights of the norms over the whole of q and of k, p2 key pages, p3 value pages, p4, p5 the pooled
+                      // blocks' pages; i0 heads, i1 kv heads, i2 d, i3 dv, i4 page size, i5 window, i6 keys a pooled block, i7 cache group;
+                      // f0 eps, f1 scale, f2 what multiplies the result -> out, at column i11 (heads * dv wide)
+  kOpDeltaRule = 21,  // linear attention by the generalized delta rule. in: projections, the columns i3 r, i4 k, i5 v, i6 gate, i7 a
+                      // (heads * d each), i8 the decay's inner projection (i2 wide); p0 the decay's outer weight [heads * d, i2], p1 its
+                      // bias, p2 the bias of a, p3 weight of the output norm (float32 [heads * d] each), p4 state rows [slots, heads, d, d];
+                      // i0 heads, i1 d; f0 eps, f1 the decay's coefficient, f2 what multiplies the result -> out, at column i9
 };
 // kOpLinearDelta i2: the result stays pending whatever the step's size (no product adds itself to the stream).
 // kOpAttention beyond i12: i13 every (0: none) and f2 coef of a temperature on the queries, 1 + coef * ln(floor((position + 1) / every)

@@ -157,6 +157,24 @@ int me_gemm_bf16_tiled(const void* X, const void* W, void* C, int M, int N, int 
                        hipStream_t stream);
 int me_gemm_bf16_library(const void* X, const void* W, void* C, int M, int N, int K, int out_dtype, hipStream_t stream);
 int me_gemm_bf16_library_add(const void* X, const void* W, float* C, int M, int N, int K, hipStream_t stream);
+int me_routed_ff_scored(const void* h, const float* Wr, const void* W_gu, const void* W_down, float* parts, void* workspace,
+                        int num_tokens, int hidden, int E, int top, int ff, int act, float limit, int scoring, int n_groups,
+                        int keep_groups, float route_scale, float* shared_gate, int dtype, hipStream_t stream);
+int me_gated_rows(const void* gu, const float* row_gate, void* act_out, int num_tokens, int ff, int act, float limit, int dtype,
+                  hipStream_t stream);
+int me_attention_general_pooled(const void* q, const void* k_cache, const void* v_cache, const int* positions, const int* token_item,
+                                const int* block_table, int table_width, void* out, int num_tokens, int nh, int nkv, int d, int dv,
+                                int bs, int window, int keep_first, const float* unturn, int un_pairing, float scale, const float* sink,
+                                const void* gate, long long gate_row, const void* k_pool, const void* v_pool, int pool,
+                                long long out_row, int out_col, float out_scale, int dtype, int items, hipStream_t stream);
+int me_whole_norm_scatter(const void* proj, long long row, int c_q, int c_k, int c_v, const float* q_w, const float* k_w,
+                          const int* positions, const int* token_item, const int* block_table, int table_width, void* q_out,
+                          void* k_cache, void* v_cache, void* k_pool, void* v_pool, int num_tokens, int nh, int nkv, int d, int dv,
+                          int bs, int pool, float eps, int dtype, hipStream_t stream);
+int me_delta_rule(const void* proj, long long row, int c_r, int c_k, int c_v, int c_g, int c_a, int c_w1, const void* W2,
+                  const float* w0, const float* a_bias, const float* norm_w, float* state, const int* item_start,
+                  const int* state_slots, void* out, long long out_row, int out_col, float out_scale, int num_tokens, int items,
+                  int heads, int d, int lora, float eps, float decay_coef, int dtype, hipStream_t stream);
 int me_sample_chunks(int vocab);
 int me_sample(const float* logits, int num_rows, int vocab, const float* temperatures, const uint64_t* keys, int* out,
               void* workspace, hipStream_t stream);

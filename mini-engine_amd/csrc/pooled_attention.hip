@@ -1,0 +1,116 @@
+// What attention over a sliding window with pooled blocks needs before its scores: the queries and keys normed over their
+// whole projection, the page writes, and the means of whole blocks of keys and values.
+//
+//   scatter   a block a token: q (all heads' nh * d elements at once) and k (nkv * d) are each divided by the root mean square
+//             of the whole row and multiplied by a weight of the row's size; the normed keys go to the key pages. The values
+//             are the keys as projected (before the norm) when no column of values is given, else that column's nkv * dv
+//             elements; they go to the value pages (transposed).
+//   pool      block b of an item holds the positions b P .. b P + P - 1. The token at position b P + P - 1 completes it: for
+//             every token of the step that completes a block, the mean of the block's P keys as the pages hold them and the
+//             mean of its P values are written to the pooled pages, at entry b: page table[b / bs], slot b % bs, the same
+//             layouts as the pages of tokens. A block may have begun in an earlier step: its keys are read from the pages.
+//             The sum runs in ascending position, so a block's mean does not depend on how the sequence was cut.
+//
+// Layouts: keys K[page, kv_head, slot, d]; values transposed V[page, kv_head, dv, slot]; pooled pages alike.
+#include "common.h"
+
+template <typename T>
+__global__ __launch_bounds__(256) void whole_norm_scatter_kernel(
+    const T* __restrict__ proj, long long row, int c_q, int c_k, int c_v, const float* __restrict__ q_w, const float* __restrict__ k_w,
+    const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table, int table_width,
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int nh, int nkv, int d, int dv, int bs, float eps) {
+  __shared__ float red[16];
+  const int t = blockIdx.x;
+  const T* p = proj + (size_t)t * row;
+  const int nq = nh * d, nk = nkv * d;
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) {
+    const float x = to_float(p[c_q + i]);
+    sq = fmaf(x, x, sq);
+  }
+  for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+    const float x = to_float(p[c_k + i]);
+    sk = fmaf(x, x, sk);
+  }
+  const float rq = rsqrtf(block_sum(sq, red) / (float)nq + eps);
+  const float rk = rsqrtf(block_sum(sk, red) / (float)nk + eps);
+  T* qo = q_out + (size_t)t * nq;
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) qo[i] = from_float<T>(to_float(p[c_q + i]) * rq * q_w[i]);
+  const int pos = positions[t];
+  const int page = block_table[(size_t)token_item[t] * table_width + pos / bs], slot = pos % bs;
+  for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+    const int kvh = i / d, e = i % d;
+    k_cache[(((size_t)page * nkv + kvh) * bs + slot) * d + e] = from_float<T>(to_float(p[c_k + i]) * rk * k_w[i]);
+  }
+  const int vcol = c_v >= 0 ? c_v : c_k;  // the values: a column of their own, or the keys as projected
+  for (int i = threadIdx.x; i < nkv * dv; i += blockDim.x) {
+    const int kvh = i / dv, e = i % dv;
+    v_cache[(((size_t)page * nkv + kvh) * dv + e) * bs + slot] = p[vcol + i];
+  }
+}
+
+// Grid (tokens, kv heads): the block of a token that completes no pooled block returns at once.
+template <typename T>
+__global__ __launch_bounds__(256) void pool_blocks_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                                                          T* __restrict__ k_pool, T* __restrict__ v_pool,
+                                                          const int* __restrict__ positions, const int* __restrict__ token_item,
+                                                          const int* __restrict__ block_table, int table_width, int nkv, int d, int dv,
+                                                          int bs, int pool) {
+  const int t = blockIdx.x, kvh = blockIdx.y;
+  const int pos = positions[t];
+  if ((pos + 1) % pool) return;
+  const int b = pos / pool, first = b * pool;
+  const int* table = block_table + (size_t)token_item[t] * table_width;
+  const int to_page = table[b / bs], to_slot = b % bs;
+  const float inv = 1.f / (float)pool;
+  for (int e = threadIdx.x; e < d + dv; e += blockDim.x) {
+    float sum = 0.f;
+    if (e < d) {
+      for (int j = 0; j < pool; ++j) {
+        const int key = first + j;
+        sum += to_float(k_cache[(((size_t)table[key / bs] * nkv + kvh) * bs + key % bs) * d + e]);
+      }
+      k_pool[(((size_t)to_page * nkv + kvh) * bs + to_slot) * d + e] = from_float<T>(sum * inv);
+    } else {
+      const int ev = e - d;
+      for (int j = 0; j < pool; ++j) {
+        const int key = first + j;
+        sum += to_float(v_cache[(((size_t)table[key / bs] * nkv + kvh) * dv + ev) * bs + key % bs]);
+      }
+      v_pool[(((size_t)to_page * nkv + kvh) * dv + ev) * bs + to_slot] = from_float<T>(sum * inv);
+    }
+  }
+}
+
+// proj [T, row]: queries at column c_q (nh * d), keys at c_k (nkv * d), values at c_v (nkv * dv; c_v < 0: the values are the
+// keys as projected, dv == d). q_w float32 [nh * d], k_w float32 [nkv * d]. pool > 0: the pooled pages get the blocks that
+// the step's tokens complete.
+extern "C" int me_whole_norm_scatter(const void* proj, long long row, int c_q, int c_k, int c_v, const float* q_w, const float* k_w,
+                                     const int* positions, const int* token_item, const int* block_table, int table_width,
+                                     void* q_out, void* k_cache, void* v_cache, void* k_pool, void* v_pool, int num_tokens, int nh,
+                                     int nkv, int d, int dv, int bs, int pool, float eps, int dtype, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (nh <= 0 || nkv <= 0 || nkv > 65535 || d <= 0 || dv <= 0 || bs <= 0 || table_width <= 0 || pool < 0)
+    return me_fail("me_whole_norm_scatter: nh=%d nkv=%d d=%d dv=%d bs=%d pool=%d", nh, nkv, d, dv, bs, pool);
+  if (c_v < 0 && dv != d) return me_fail("me_whole_norm_scatter: values that are the keys have the keys' size, not %d", dv);
+  if (c_q < 0 || c_q + (long long)nh * d > row || c_k < 0 || c_k + (long long)nkv * d > row ||
+      (c_v >= 0 && c_v + (long long)nkv * dv > row))
+    return me_fail("me_whole_norm_scatter: columns %d, %d, %d of a row of %lld", c_q, c_k, c_v, row);
+  if (pool > 0 && (!k_pool || !v_pool)) return me_fail("me_whole_norm_scatter: pooled blocks need pages of their own");
+#define WN_RUN(TT)                                                                                                                \
+  do {                                                                                                                            \
+    whole_norm_scatter_kernel<TT><<<num_tokens, 256, 0, stream>>>((const TT*)proj, row, c_q, c_k, c_v, q_w, k_w, positions,        \
+                                                                  token_item, block_table, table_width, (TT*)q_out, (TT*)k_cache, \
+                                                                  (TT*)v_cache, nh, nkv, d, dv, bs, eps);                         \
+    if (pool > 0)                                                                                                                 \
+      pool_blocks_kernel<TT><<<dim3(num_tokens, nkv), d + dv >= 256 ? 256 : 64 * ((d + dv + 63) / 64), 0, stream>>>(              \
+          (const TT*)k_cache, (const TT*)v_cache, (TT*)k_pool, (TT*)v_pool, positions, token_item, block_table, table_width, nkv, \
+          d, dv, bs, pool);                                                                                                       \
+  } while (0)
+  if (dtype == ME_F32)
+    WN_RUN(float);
+  else
+    WN_RUN(bf16_t);
+#undef WN_RUN
+  return me_check_launch("me_whole_norm_scatter");
+}

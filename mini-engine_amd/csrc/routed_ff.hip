@@ -13,22 +13,28 @@
 
 extern "C" int me_gemm_grouped_tile_rows();
 extern "C" int me_gemm_grouped_bf16(const void* X, const void* W, const int* plan, const int* sorted, const float* wts, void* acts,
-                                    float* parts, int num_tokens, int N, int K, int top, int max_tiles, int gated, hipStream_t stream);
+                                    float* parts, int num_tokens, int N, int K, int top, int max_tiles, int gated, float limit,
+                                    hipStream_t stream);
 
 #define RF_MAX_EXPERTS 1024
 #define RF_MAX_TOP 32
+#define RF_SCORE_SOFTMAX 0  // the picks' weights: the softmax over the picked logits
+#define RF_SCORE_SIGMOID 1  // the picks' scores sigmoid(z) over their sum (+ 1e-20), times a scale; picks bounded by groups
 #define RF_DIRECT_PAIRS 16  // steps of up to this many pairs (token, pick) are not sorted: a pair is a tile
 
 template <typename T>
 __global__ __launch_bounds__(1024) void routed_route_kernel(const T* __restrict__ h, const float* __restrict__ Wr, int* __restrict__ ids,
                                                             float* __restrict__ wts, int hidden, int E, int top,
-                                                            int* __restrict__ plan, int* __restrict__ sorted, int num_pairs) {
-  __shared__ float z[RF_MAX_EXPERTS];
+                                                            int* __restrict__ plan, int* __restrict__ sorted, int num_pairs,
+                                                            int scoring, int n_groups, int keep_groups, float route_scale,
+                                                            float* __restrict__ shared_gate) {
+  __shared__ float z[RF_MAX_EXPERTS + 1], sc[RF_MAX_EXPERTS], gs[RF_MAX_EXPERTS];
   const int t = blockIdx.x, wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const T* row = h + (size_t)t * hidden;
   // a wave an expert at a time; a lane's elements lie 64 apart, four of them in flight together with sums of their own
   const int waves = blockDim.x / ME_WAVE;
-  for (int e = wave; e < E; e += waves) {
+  const int logits = E + (shared_gate ? 1 : 0);  // (the row behind the experts': the gate of an expert that every token uses)
+  for (int e = wave; e < logits; e += waves) {
     const float* w = Wr + (size_t)e * hidden;
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     int c = lane;
@@ -44,6 +50,48 @@ __global__ __launch_bounds__(1024) void routed_route_kernel(const T* __restrict_
   }
   __syncthreads();
   if (wave != 0) return;
+  if (shared_gate && lane == 0) shared_gate[t] = 1.f / (1.f + expf(-z[E]));
+  if (scoring == RF_SCORE_SIGMOID) {
+    // scores sigmoid(z); the experts form n_groups equal groups of neighbours, a group's score is the sum of its two largest
+    // scores, and only experts of the keep_groups best groups can be picked (the lower index among equals, as for the picks)
+    for (int e = lane; e < E; e += ME_WAVE) sc[e] = 1.f / (1.f + expf(-z[e]));
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    if (n_groups > 1 && keep_groups < n_groups) {
+      const int per = E / n_groups;
+      for (int g = lane; g < n_groups; g += ME_WAVE) {
+        float a = -INFINITY, b = -INFINITY;  // the largest and the second largest
+        for (int i = 0; i < per; ++i) {
+          const float v = sc[g * per + i];
+          if (v > a) b = a, a = v;
+          else if (v > b) b = v;
+        }
+        gs[g] = per > 1 ? a + b : a;
+      }
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      for (int j = 0; j < keep_groups; ++j) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+        for (int g = lane; g < n_groups; g += ME_WAVE)
+          if (gs[g] > best) best = gs[g], at = g;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+          const float ob = __shfl_xor(best, off, ME_WAVE);
+          const int oa = __shfl_xor(at, off, ME_WAVE);
+          if (ob > best || (ob == best && oa < at)) best = ob, at = oa;
+        }
+        if (at >= n_groups) break;  // (a row of NaNs)
+        if (lane == 0) gs[at] = -INFINITY;  // taken: its experts stay
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+      }
+      for (int e = lane; e < E; e += ME_WAVE)
+        if (gs[e / per] != -INFINITY) z[e] = -INFINITY;  // a group that was not taken
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+    }
+  }
   float mine = 0.f, zmax = 0.f, sum = 0.f;  // lane j keeps the weight of the j-th pick
   int mine_e = 0;
   for (int j = 0; j < top; ++j) {
@@ -59,7 +107,8 @@ __global__ __launch_bounds__(1024) void routed_route_kernel(const T* __restrict_
     }
     if (at >= E) at = 0;  // (a row of NaNs, as rows that pad a replayed step may be: any expert)
     if (j == 0) zmax = best;
-    const float p = expf(best - zmax);
+    // the pick's weight before it is divided by the picks' sum: exp(z - z_max), or the pick's score
+    const float p = scoring == RF_SCORE_SIGMOID ? sc[at] : expf(best - zmax);
     if (lane == j) mine = p, mine_e = at;
     sum += p;
     if (lane == 0) {
@@ -69,7 +118,7 @@ __global__ __launch_bounds__(1024) void routed_route_kernel(const T* __restrict_
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
-  if (lane < top) wts[(size_t)t * top + lane] = mine / sum;
+  if (lane < top) wts[(size_t)t * top + lane] = scoring == RF_SCORE_SIGMOID ? mine / (sum + 1e-20f) * route_scale : mine / sum;
   // A step of very few pairs needs no sorting: every pair is a tile of its own, in the order of the pairs (plan and
   // sorted as routed_sort_kernel leaves them for tiles of one row).
   if (plan && lane < top) {
@@ -113,7 +162,7 @@ __global__ __launch_bounds__(1024) void routed_sort_kernel(const int* __restrict
 template <typename T>
 __global__ __launch_bounds__(256) void routed_gate_up_kernel(const T* __restrict__ h, const T* __restrict__ W_gu,
                                                              const int* __restrict__ plan, const int* __restrict__ sorted,
-                                                             T* __restrict__ acts, int hidden, int ff, int top, int act) {
+                                                             T* __restrict__ acts, int hidden, int ff, int top, int act, float limit) {
   __shared__ TileLds lds;
   const int tile = blockIdx.x;
   if (tile >= plan[0]) return;
@@ -129,7 +178,7 @@ __global__ __launch_bounds__(256) void routed_gate_up_kernel(const T* __restrict
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int row = ty + 4 * i;
-    if (row < rows) acts[(size_t)(begin + row) * ff + c0 + tx] = from_float<T>(gate_act(g[i], act) * u[i]);
+    if (row < rows) acts[(size_t)(begin + row) * ff + c0 + tx] = from_float<T>(gated_pair(g[i], u[i], act, limit));
   }
 }
 
@@ -168,7 +217,7 @@ __global__ __launch_bounds__(256) void routed_tile_mfma_kernel(const bf16_t* __r
                                                                const int* __restrict__ plan, const int* __restrict__ sorted,
                                                                const float* __restrict__ wts, bf16_t* __restrict__ acts,
                                                                float* __restrict__ parts, int num_tokens, int N, int K, int top,
-                                                               int act) {
+                                                               int act, float limit) {
   const int tile = blockIdx.x;
   if (tile >= plan[0]) return;
   const int e = plan[1 + 3 * tile], begin = plan[2 + 3 * tile], rows = plan[3 + 3 * tile];
@@ -199,7 +248,7 @@ __global__ __launch_bounds__(256) void routed_tile_mfma_kernel(const bf16_t* __r
       const int col = n0 + 4 * g + i;
       if (col >= N) continue;
       if (GATED)
-        acts[(size_t)(begin + row) * N + col] = from_float<bf16_t>(gate_act(acc[t][0][i], act) * acc[t][ACCS - 1][i]);
+        acts[(size_t)(begin + row) * N + col] = from_float<bf16_t>(gated_pair(acc[t][0][i], acc[t][ACCS - 1][i], act, limit));
       else
         parts[((size_t)(pair[t] % top) * num_tokens + pair[t] / top) * N + col] = wts[pair[t]] * acc[t][0][i];
     }
@@ -214,7 +263,7 @@ __global__ __launch_bounds__(256) void routed_tile_ksplit_kernel(const bf16_t* _
                                                                  const int* __restrict__ plan, const int* __restrict__ sorted,
                                                                  const float* __restrict__ wts, bf16_t* __restrict__ acts,
                                                                  float* __restrict__ parts, int num_tokens, int N, int K, int top,
-                                                                 int act) {
+                                                                 int act, float limit) {
   constexpr int ACCS = GATED ? 2 : 1, WAVES = 4, U = 2;
   __shared__ float red[WAVES][ACCS][64][4];
   const int tile = blockIdx.x;
@@ -266,7 +315,7 @@ __global__ __launch_bounds__(256) void routed_tile_ksplit_kernel(const bf16_t* _
     const int col = n0 + 4 * g + i;
     if (col >= N) continue;
     if (GATED)
-      acts[(size_t)(begin + r) * N + col] = from_float<bf16_t>(gate_act(sum[0][i], act) * sum[ACCS - 1][i]);
+      acts[(size_t)(begin + r) * N + col] = from_float<bf16_t>(gated_pair(sum[0][i], sum[ACCS - 1][i], act, limit));
     else
       parts[((size_t)(pair % top) * num_tokens + pair / top) * N + col] = wts[pair] * sum[0][i];
   }
@@ -284,9 +333,17 @@ extern "C" long long me_routed_ff_workspace(long long tokens, int E, int top, in
 }
 
 // h [T, hidden] -> parts float32 [top, T, hidden]. Wr float32 [E, hidden]; W_gu [E, 2 ff, hidden]; W_down [E, hidden, ff].
-extern "C" int me_routed_ff(const void* h, const float* Wr, const void* W_gu, const void* W_down, float* parts, void* workspace,
-                            int num_tokens, int hidden, int E, int top, int ff, int act, int dtype, hipStream_t stream) {
+// limit: what an activation with a limit clamps by. scoring (RF_SCORE_*), n_groups, keep_groups, route_scale: how the picks are
+// bounded and weighted. shared_gate (float32 [T] or null): Wr has one more row behind the experts', and the sigmoid of a
+// token's product with it is written there (the gate of an expert that every token uses).
+extern "C" int me_routed_ff_scored(const void* h, const float* Wr, const void* W_gu, const void* W_down, float* parts, void* workspace,
+                                   int num_tokens, int hidden, int E, int top, int ff, int act, float limit, int scoring, int n_groups,
+                                   int keep_groups, float route_scale, float* shared_gate, int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
+  if (scoring != RF_SCORE_SOFTMAX && scoring != RF_SCORE_SIGMOID) return me_fail("me_routed_ff: scoring %d", scoring);
+  if (scoring == RF_SCORE_SIGMOID && (n_groups < 1 || E % n_groups || keep_groups < 1 || keep_groups > n_groups ||
+                                      (long long)keep_groups * (E / n_groups) < top))
+    return me_fail("me_routed_ff: %d experts in %d groups of which %d are kept, %d picks", E, n_groups, keep_groups, top);
   if (E < 1 || E > RF_MAX_EXPERTS || top < 1 || top > RF_MAX_TOP || top > E)
     return me_fail("me_routed_ff: %d experts (at most %d), %d of them a token (at most %d)", E, RF_MAX_EXPERTS, top, RF_MAX_TOP);
   if (hidden <= 0 || ff <= 0) return me_fail("me_routed_ff: hidden=%d ff=%d", hidden, ff);
@@ -308,59 +365,94 @@ extern "C" int me_routed_ff(const void* h, const float* Wr, const void* W_gu, co
     const int wide = P >= 32ll * E;  // 32 and more pairs an expert on average: tiles of 64 pairs
     const bool direct = P <= RF_DIRECT_PAIRS && (ff + 15) / 16 <= 65535 && (hidden + 15) / 16 <= 65535;
     routed_route_kernel<bf16_t><<<num_tokens, route_threads, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top,
-                                                                            direct ? plan : nullptr, direct ? sorted : nullptr, (int)P);
+                                                                            direct ? plan : nullptr, direct ? sorted : nullptr, (int)P,
+                                                                            scoring, n_groups, keep_groups, route_scale, shared_gate);
     if (direct) {  // the router has written the list of tiles itself
       const dim3 k_up((unsigned)P, (ff + 15) / 16), k_down((unsigned)P, (hidden + 15) / 16);
       routed_tile_ksplit_kernel<true><<<k_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, wts, (bf16_t*)acts,
-                                                                nullptr, num_tokens, ff, hidden, top, act);
+                                                                nullptr, num_tokens, ff, hidden, top, act, limit);
       routed_tile_ksplit_kernel<false><<<k_down, 256, 0, stream>>>((const bf16_t*)acts, (const bf16_t*)W_down, plan, sorted, wts, nullptr,
-                                                                 parts, num_tokens, hidden, ff, top, act);
+                                                                 parts, num_tokens, hidden, ff, top, act, limit);
       return me_check_launch("me_routed_ff");
     }
     if (P >= 96ll * E && hidden % 64 == 0 && ff % 64 == 0) {
       // prompts: tiles of 128 pairs through the product that stages both operands in LDS (gemm_grouped.hip)
       const int rows128 = me_gemm_grouped_tile_rows(), tiles128 = (int)((P + rows128 - 1) / rows128) + E;
       routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, rows128, plan, sorted);
-      if (me_gemm_grouped_bf16(h, W_gu, plan, sorted, wts, acts, nullptr, num_tokens, ff, hidden, top, tiles128, act, stream)) return 1;
-      return me_gemm_grouped_bf16(acts, W_down, plan, sorted, wts, nullptr, parts, num_tokens, hidden, ff, top, tiles128, 0, stream);
+      if (me_gemm_grouped_bf16(h, W_gu, plan, sorted, wts, acts, nullptr, num_tokens, ff, hidden, top, tiles128, act, limit, stream)) return 1;
+      return me_gemm_grouped_bf16(acts, W_down, plan, sorted, wts, nullptr, parts, num_tokens, hidden, ff, top, tiles128, 0, 0.f, stream);
     }
     routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, wide ? 64 : 16, plan, sorted);
     if (wide) {
       const unsigned tiles64 = (unsigned)((P + 63) / 64) + E;  // fewer tiles than the list's bound: whole blocks that only return
       const dim3 g_up(tiles64, (ff + TP_COLS - 1) / TP_COLS), g_down(tiles64, (hidden + TP_COLS - 1) / TP_COLS);
       routed_tile_mfma_kernel<4, true><<<g_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, wts, (bf16_t*)acts,
-                                                                 nullptr, num_tokens, ff, hidden, top, act);
+                                                                 nullptr, num_tokens, ff, hidden, top, act, limit);
       routed_tile_mfma_kernel<4, false><<<g_down, 256, 0, stream>>>((const bf16_t*)acts, (const bf16_t*)W_down, plan, sorted, wts, nullptr,
-                                                                  parts, num_tokens, hidden, ff, top, act);
+                                                                  parts, num_tokens, hidden, ff, top, act, limit);
     } else if (P <= 4ll * E && (ff + 15) / 16 <= 65535 && (hidden + 15) / 16 <= 65535) {
       // few pairs (decode steps): most tiles hold a pair or two, and what a step waits for is the walk over k
       const dim3 k_up(max_tiles, (ff + 15) / 16), k_down(max_tiles, (hidden + 15) / 16);
       routed_tile_ksplit_kernel<true><<<k_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, wts, (bf16_t*)acts,
-                                                                nullptr, num_tokens, ff, hidden, top, act);
+                                                                nullptr, num_tokens, ff, hidden, top, act, limit);
       routed_tile_ksplit_kernel<false><<<k_down, 256, 0, stream>>>((const bf16_t*)acts, (const bf16_t*)W_down, plan, sorted, wts, nullptr,
-                                                                 parts, num_tokens, hidden, ff, top, act);
+                                                                 parts, num_tokens, hidden, ff, top, act, limit);
     } else {
       routed_tile_mfma_kernel<1, true><<<g_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, wts, (bf16_t*)acts,
-                                                                 nullptr, num_tokens, ff, hidden, top, act);
+                                                                 nullptr, num_tokens, ff, hidden, top, act, limit);
       routed_tile_mfma_kernel<1, false><<<g_down, 256, 0, stream>>>((const bf16_t*)acts, (const bf16_t*)W_down, plan, sorted, wts, nullptr,
-                                                                  parts, num_tokens, hidden, ff, top, act);
+                                                                  parts, num_tokens, hidden, ff, top, act, limit);
     }
     return me_check_launch("me_routed_ff");
   }
   if (dtype == ME_F32) {
-    routed_route_kernel<float><<<num_tokens, route_threads, 0, stream>>>((const float*)h, Wr, ids, wts, hidden, E, top, nullptr, nullptr, 0);
+    routed_route_kernel<float><<<num_tokens, route_threads, 0, stream>>>((const float*)h, Wr, ids, wts, hidden, E, top, nullptr, nullptr, 0,
+                                                                         scoring, n_groups, keep_groups, route_scale, shared_gate);
     routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, TP_ROWS, plan, sorted);
     routed_gate_up_kernel<float><<<g_up, 256, 0, stream>>>((const float*)h, (const float*)W_gu, plan, sorted, (float*)acts, hidden, ff,
-                                                            top, act);
+                                                            top, act, limit);
     routed_down_kernel<float><<<g_down, 256, 0, stream>>>((const float*)acts, (const float*)W_down, plan, sorted, wts, parts,
                                                           num_tokens, hidden, ff, top);
   } else {
-    routed_route_kernel<bf16_t><<<num_tokens, route_threads, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top, nullptr, nullptr, 0);
+    routed_route_kernel<bf16_t><<<num_tokens, route_threads, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top, nullptr, nullptr, 0,
+                                                                          scoring, n_groups, keep_groups, route_scale, shared_gate);
     routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, TP_ROWS, plan, sorted);
     routed_gate_up_kernel<bf16_t><<<g_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, (bf16_t*)acts, hidden,
-                                                             ff, top, act);
+                                                             ff, top, act, limit);
     routed_down_kernel<bf16_t><<<g_down, 256, 0, stream>>>((const bf16_t*)acts, (const bf16_t*)W_down, plan, sorted, wts, parts,
                                                            num_tokens, hidden, ff, top);
   }
   return me_check_launch("me_routed_ff");
+}
+
+extern "C" int me_routed_ff(const void* h, const float* Wr, const void* W_gu, const void* W_down, float* parts, void* workspace,
+                            int num_tokens, int hidden, int E, int top, int ff, int act, int dtype, hipStream_t stream) {
+  return me_routed_ff_scored(h, Wr, W_gu, W_down, parts, workspace, num_tokens, hidden, E, top, ff, act, 0.f, RF_SCORE_SOFTMAX, 1, 1,
+                             1.f, nullptr, dtype, stream);
+}
+
+// An expert that every token uses, behind its ungated product: gu [T, 2 ff] (gate columns, then up columns) ->
+// act [T, ff] = gated_pair(gate, up) * row_gate[t] (row_gate float32 [T] or null: 1).
+template <typename T>
+__global__ __launch_bounds__(256) void gated_rows_kernel(const T* __restrict__ gu, const float* __restrict__ row_gate,
+                                                         T* __restrict__ act_out, long long total, int ff, int act, float limit) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long long t = i / ff;
+  const int c = (int)(i % ff);
+  const float g = to_float(gu[t * 2 * ff + c]), u = to_float(gu[t * 2 * ff + ff + c]);
+  const float y = gated_pair(g, u, act, limit) * (row_gate ? row_gate[t] : 1.f);
+  act_out[i] = from_float<T>(y);
+}
+
+extern "C" int me_gated_rows(const void* gu, const float* row_gate, void* act_out, int num_tokens, int ff, int act, float limit, int dtype,
+                             hipStream_t stream) {
+  if (num_tokens <= 0 || ff <= 0) return 0;
+  const long long total = (long long)num_tokens * ff;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (dtype == ME_F32)
+    gated_rows_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, row_gate, (float*)act_out, total, ff, act, limit);
+  else
+    gated_rows_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, row_gate, (bf16_t*)act_out, total, ff, act, limit);
+  return me_check_launch("me_gated_rows");
 }

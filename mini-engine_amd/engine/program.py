@@ -29,7 +29,8 @@ _vp, _i64, _i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 _declared = False
 
 (EMBED, NORM_LINEAR, NORM, LINEAR, LINEAR_DELTA, DELTA, ATTENTION, HEAD, SAMPLE, ADD, CALL, HEAD_ROWS, DECAY_STATE, HOLD, STREAMS,
- STREAM_NORM, STREAM_HEAD, LATENT_ATTENTION, ROUTED_FF, STREAM_NORM_LINEAR) = range(20)
+ STREAM_NORM, STREAM_HEAD, LATENT_ATTENTION, ROUTED_FF, STREAM_NORM_LINEAR, POOLED_ATTENTION, DELTA_RULE) = range(22)
+ROUTER_SCORINGS = {"softmax_picked": 0, "sigmoid_normalized": 1}  # csrc/routed_ff.hip: RF_SCORE_*
 OP_PTRS, OP_INTS, OP_FLOATS = 8, 16, 4  # csrc/host/program.h: kOpPtrs, kOpInts, kOpFloats
 MAX_STREAMS = 8  # csrc/streams.hip: ME_MAX_STREAMS
 _RAISES = {1: ValueError, 2: RuntimeError, 3: AssertionError}
@@ -159,6 +160,16 @@ class StreamNormed:
         return self._value
 
 
+class NormedValue:
+    """Normed activations that are a value already, with the face of :class:`Normed`."""
+
+    def __init__(self, value: int):
+        self._value, self.used = value, True
+
+    def value(self) -> int:
+        return self._value
+
+
 class StepProgram:
     def __init__(self, dtype: torch.dtype, hidden: int, vocab: int, max_positions: int):
         self._L = _api()
@@ -176,6 +187,9 @@ class StepProgram:
         self._held_value: int | None = None  # the value of a delta that was set aside (hold)
         self.num_ops = 0
         self.delta_scale = 1.0  # what the block being written multiplies its parts' results by (set by the block)
+        # a part's result must wait for the next add whatever the step's size: the block reads the stream once more before it
+        # (no product adds itself into the stream)
+        self.delta_stays = False
         self.num_streams = 0  # residual streams of a token (0: the one plain stream)
         self._stream_rewrite: torch.Tensor | None = None  # how the pending result rewrites the streams (mix, then out)
         self.draws = False
@@ -279,7 +293,7 @@ class StepProgram:
             x.used = True
             self.pending_consumed()
             return out
-        src = x.value() if isinstance(x, (Normed, CalledNorm, StreamNormed)) else x
+        src = x.value() if isinstance(x, (Normed, CalledNorm, StreamNormed, NormedValue)) else x
         if self._value_kinds[src][0] != k:
             raise ValueError(f"the weight reads {k} columns, the value has {self._value_kinds[src][0]}")
         self.op(LINEAR, in_=src, out=out, ptrs=[None, weight], ints=[rows, k, gate])
@@ -290,7 +304,7 @@ class StepProgram:
         rows, k = weight.shape
         self._want(weight, self.dtype, (self.hidden, self._value_kinds[x][0]), "weight")
         out = self.take(rows)
-        self.op(LINEAR_DELTA, in_=x, out=out, ptrs=[None, weight], ints=[rows, k], floats=[self.delta_scale])
+        self.op(LINEAR_DELTA, in_=x, out=out, ptrs=[None, weight], ints=[rows, k, int(self.delta_stays)], floats=[self.delta_scale])
         self._pending_value = out
 
     def delta(self, x: int) -> None:
@@ -371,22 +385,109 @@ class StepProgram:
                 ints=[heads, head_dim, rotary_dim, rank, value_dim, block_size, group, rope.shape[0], value_rows], floats=[eps, scale])
         return out
 
-    def routed_ff(self, x: int, *, router: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, top_k: int, activation: str) -> None:
+    def routed_ff(self, x: int, *, router: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, top_k: int, activation: str,
+                  activation_limit: float = 0.0, scoring: str = "softmax_picked", num_groups: int = 1, keep_groups: int = 1,
+                  route_scale: float = 1.0, shared_gate_up: torch.Tensor | None = None, shared_down: torch.Tensor | None = None,
+                  shared_limit: float = 0.0) -> None:
         """A feed-forward of routed experts on the value ``x`` as the part's result. ``router`` float32 ``[experts, hidden]``;
         ``gate_up`` ``[experts, 2 ff, hidden]`` (an expert's gate rows, then its up rows) and ``down`` ``[experts, hidden, ff]``
-        in the compute dtype."""
+        in the compute dtype. ``scoring``, ``num_groups``, ``keep_groups``, ``route_scale``: how the picks are bounded and weighted
+        (:class:`~mini_engine_amd.config.specs.RoutedExpertsSpec`). ``shared_gate_up`` ``[2 ff_s, hidden]`` and ``shared_down``
+        ``[hidden, ff_s]``: an expert that every token uses; the router then has one more row behind the experts', the token's
+        product with which, through a sigmoid, multiplies that expert's result."""
         from ..ops.kernels import gate_code
 
         experts, two_ff, hidden = gate_up.shape
         if self._value_kinds[x] != (self.hidden, self.elem) or hidden != self.hidden:
             raise ValueError("routed experts read the hidden size in the compute dtype")
-        self._want(router, torch.float32, (experts, hidden), "router")
+        shared_ff = 0
+        if shared_gate_up is not None:
+            shared_ff = shared_gate_up.shape[0] // 2
+            self._want(shared_gate_up, self.dtype, (2 * shared_ff, hidden), "the shared expert's gate and up rows")
+            self._want(shared_down, self.dtype, (hidden, shared_ff), "the shared expert's down rows")
+        self._want(router, torch.float32, (experts + (1 if shared_ff else 0), hidden), "router")
         self._want(gate_up, self.dtype, None, "experts' gate and up rows")
         self._want(down, self.dtype, (experts, hidden, two_ff // 2), "experts' down rows")
         if not 1 <= top_k <= experts:
             raise ValueError(f"{top_k} of {experts} experts a token")
-        self.op(ROUTED_FF, in_=x, ptrs=[router, gate_up, down], ints=[experts, top_k, two_ff // 2, gate_code(activation)])
+        if scoring not in ROUTER_SCORINGS:
+            raise ValueError(f"a router scores by one of {sorted(ROUTER_SCORINGS)}, not {scoring!r}")
+        if num_groups < 1 or experts % num_groups or not 1 <= keep_groups <= num_groups or keep_groups * (experts // num_groups) < top_k:
+            raise ValueError(f"{experts} experts in {num_groups} groups of which {keep_groups} are kept, {top_k} picks")
+        self.op(ROUTED_FF, in_=x, ptrs=[router, gate_up, down, shared_gate_up, shared_down],
+                ints=[experts, top_k, two_ff // 2, gate_code(activation, limited=True), ROUTER_SCORINGS[scoring], num_groups, keep_groups, shared_ff],
+                floats=[activation_limit, route_scale, shared_limit, self.delta_scale])
         self._pending_value = None
+
+    def normed_again(self, norm) -> NormedValue:
+        """A second norm of the residual stream as the norm before left it (an RMS-shaped norm, in groups or not): nothing is
+        pending, and a result that was set aside stays aside. Returns the value of the normed activations."""
+        weight, eps = norm.as_fused()
+        self._want(weight, torch.float32, (self.hidden,), "norm weight")
+        if self._pending_value is not None:
+            raise ValueError("a result is pending before a second norm of the stream")
+        out = self.take(self.hidden, self.elem)
+        self.op(NORM, out=out, ptrs=[weight], ints=[getattr(norm, "groups", 1), 1], floats=[eps])
+        return NormedValue(out)
+
+    def pooled_attention(self, proj: int, out: int, *, q_col: int, k_col: int, v_col: int, out_col: int, q_norm: torch.Tensor,
+                         k_norm: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, k_pool: torch.Tensor | None,
+                         v_pool: torch.Tensor | None, heads: int, kv_heads: int, head_dim: int, value_dim: int, block_size: int,
+                         window: int, pooled_block: int, group: int, eps: float, scale: float, out_scale: float = 1.0) -> None:
+        """Causal attention without rotation whose q and k are normed over their whole projection, over a window of ``window``
+        keys (0: all) and, with ``pooled_block`` P > 0, the means of the whole blocks of P keys and values before the window. The
+        value ``proj`` holds the queries at column ``q_col``, the keys at ``k_col`` and the values at ``v_col`` (-1: the values are
+        the keys as projected); the result (``heads * value_dim`` columns, times ``out_scale``) goes to the value ``out`` at
+        column ``out_col``."""
+        row, out_row = self._value_kinds[proj][0], self._value_kinds[out][0]
+        if self._value_kinds[proj][1] != self.elem or self._value_kinds[out][1] != self.elem:
+            raise ValueError("attention reads and writes values of the compute dtype")
+        for col, n in ((q_col, heads * head_dim), (k_col, kv_heads * head_dim)) + (((v_col, kv_heads * value_dim),) if v_col >= 0 else ()):
+            if col < 0 or col + n > row:
+                raise ValueError(f"columns {col} .. {col + n - 1} of a value of {row}")
+        if out_col < 0 or out_col + heads * value_dim > out_row:
+            raise ValueError(f"the result at column {out_col} of a value of {out_row}")
+        if v_col < 0 and value_dim != head_dim:
+            raise ValueError("values that are the keys have the keys' size")
+        self._want(q_norm, torch.float32, (heads * head_dim,), "weight of the queries' norm")
+        self._want(k_norm, torch.float32, (kv_heads * head_dim,), "weight of the keys' norm")
+        pages = int(k_cache.shape[0])
+        for t, shape, what in ((k_cache, (pages, kv_heads, block_size, head_dim), "key pages"),
+                               (v_cache, (pages, kv_heads, value_dim, block_size), "value pages")):
+            self._want(t, self.dtype, shape, what)
+        if pooled_block:
+            if window <= 0:
+                raise ValueError("pooled blocks lie before a window")
+            self._want(k_pool, self.dtype, tuple(k_cache.shape), "pooled key pages")
+            self._want(v_pool, self.dtype, tuple(v_cache.shape), "pooled value pages")
+        self.op(POOLED_ATTENTION, in_=proj, out=out, ptrs=[q_norm, k_norm, k_cache, v_cache, k_pool, v_pool],
+                ints=[heads, kv_heads, head_dim, value_dim, block_size, window, pooled_block, group, q_col, k_col, v_col, out_col],
+                floats=[eps, scale, out_scale])
+
+    def delta_rule(self, proj: int, out: int, *, cols: dict, out_col: int, decay_outer: torch.Tensor, decay_bias: torch.Tensor,
+                   rate_bias: torch.Tensor, norm_weight: torch.Tensor, state: torch.Tensor, heads: int, head_dim: int,
+                   decay_rank: int, eps: float, decay_coef: float, out_scale: float = 1.0) -> None:
+        """Linear attention by the generalized delta rule over the step's items, from and into their rows of ``state``
+        ``[slots, heads, head_dim, head_dim]`` (float32). ``cols`` gives the columns of the value ``proj`` at which r, k, v, the
+        gate ``g`` and the removal rate ``a`` (``heads * head_dim`` wide each) and the decay's inner projection ``w1``
+        (``decay_rank`` wide) begin; the result (times ``out_scale``) goes to the value ``out`` at column ``out_col``."""
+        row, out_row = self._value_kinds[proj][0], self._value_kinds[out][0]
+        n = heads * head_dim
+        if self._value_kinds[proj][1] != self.elem or self._value_kinds[out][1] != self.elem:
+            raise ValueError("the delta rule reads and writes values of the compute dtype")
+        for role in ("r", "k", "v", "g", "a", "w1"):
+            width = decay_rank if role == "w1" else n
+            if cols[role] < 0 or cols[role] + width > row:
+                raise ValueError(f"{role}: columns {cols[role]} .. {cols[role] + width - 1} of a value of {row}")
+        if out_col < 0 or out_col + n > out_row:
+            raise ValueError(f"the result at column {out_col} of a value of {out_row}")
+        self._want(decay_outer, self.dtype, (n, decay_rank), "the decay's outer weight")
+        for t, what in ((decay_bias, "the decay's bias"), (rate_bias, "the removal rate's bias"), (norm_weight, "weight of the output norm")):
+            self._want(t, torch.float32, (n,), what)
+        self._want(state, torch.float32, (state.shape[0], heads, head_dim, head_dim), "state")
+        self.op(DELTA_RULE, in_=proj, out=out, ptrs=[decay_outer, decay_bias, rate_bias, norm_weight, state],
+                ints=[heads, head_dim, decay_rank, cols["r"], cols["k"], cols["v"], cols["g"], cols["a"], cols["w1"], out_col],
+                floats=[eps, decay_coef, out_scale])
 
     # ----------------------------------------------------------- several residual streams
     def spread_streams(self, streams: int) -> None:

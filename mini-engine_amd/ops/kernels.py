@@ -246,12 +246,20 @@ def rmsnorm(inp: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tens
 GATE_ACTIVATIONS = {"silu": 1, "gelu_tanh": 2}  # the codes of the kernels' `gated` arguments (MeGate in csrc/common.h)
 
 
-def gate_code(gated) -> int:
-    """0 for a product that is not gated; else the code of the gate's activation. ``True`` means silu."""
+# activations that clamp by a limit: the kernels of routed experts take them (with the limit beside the code), the dense
+# products' epilogues do not
+LIMITED_GATE_ACTIVATIONS = {"clamped_sigmoid": 3}
+
+
+def gate_code(gated, limited: bool = False) -> int:
+    """0 for a product that is not gated; else the code of the gate's activation. ``True`` means silu. ``limited``: the caller's
+    kernels also take the activations with a limit."""
     if not gated:
         return 0
     if gated is True:
         return GATE_ACTIVATIONS["silu"]
+    if limited and gated in LIMITED_GATE_ACTIVATIONS:
+        return LIMITED_GATE_ACTIVATIONS[gated]
     if gated not in GATE_ACTIVATIONS:
         raise ValueError(f"unknown gate activation {gated!r}; known: {sorted(GATE_ACTIVATIONS)}")
     return GATE_ACTIVATIONS[gated]

@@ -1,6 +1,6 @@
 """Parts of a decoder layer. Importing this package registers the built-in kinds."""
 
-from . import attention, decay_state, latent_attention, mlp, norm, rotary, routed_experts  # noqa: F401
+from . import attention, decay_state, delta_rule, latent_attention, mlp, norm, pair, rotary, routed_experts  # noqa: F401
 from .base import (
     BLOCK_ARRANGEMENTS,
     FEED_FORWARDS,
@@ -12,6 +12,7 @@ from .base import (
     KVCacheNeed,
     Mixer,
     Norm,
+    PairBinding,
     PositionEncoding,
     StateBinding,
     StateNeed,
@@ -31,6 +32,7 @@ __all__ = [
     "Mixer",
     "NORMS",
     "Norm",
+    "PairBinding",
     "POSITION_ENCODINGS",
     "ParallelBlock",
     "PositionEncoding",

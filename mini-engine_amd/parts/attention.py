@@ -57,9 +57,27 @@ class Attention(Mixer):
             raise ValueError(f"a temperature on the queries grows every {self.q_temp[1]} positions: at least every one")
         self.gated = bool(getattr(s, "output_gate", False))
         self.norm_weighted = bool(getattr(s, "qk_norm_weight", True))
+        # q and k normed over their whole projection (no rotation): a form of its own, which may take its values from the keys
+        # as projected and see the means of whole blocks of keys before its window
+        self.whole = getattr(s, "qk_norm_over", "head") == "projection"
+        self.values_from_keys = bool(getattr(s, "values_from_keys", False))
+        self.pooled_block = int(getattr(s, "pooled_block", 0))
+        if getattr(s, "qk_norm_over", "head") not in ("head", "projection"):
+            raise ValueError(f"q and k are normed over 'head' or 'projection', not {s.qk_norm_over!r}")
+        if (self.values_from_keys or self.pooled_block) and not self.whole:
+            raise ValueError("values taken from the keys and pooled blocks are built for q and k normed over their whole projection")
+        if self.whole:
+            if (s.qk_norm_eps is None or self.position is not None or self.keep_first or self.value_position is not None
+                    or self.q_temp is not None or self.gated or s.cache_from is not None or not self.norm_weighted):
+                raise ValueError("attention normed over the whole projection has a weighted norm, no rotation, no kept first keys, "
+                                 "no gate, no temperature, and pages of its own")
+            if self.values_from_keys and self.dv != self.d:
+                raise ValueError(f"values that are the keys have the keys' size {self.d}, not {self.dv}")
+            if self.pooled_block < 0 or (self.pooled_block and not s.window):
+                raise ValueError(f"pooled_block={self.pooled_block} must be >= 0 and needs a window")
         # the plain form: what the matrix-core kernels and the fused decode prologue are written for
         self.plain = (self.dv == self.d and not self.keep_first and self.pairing == 0 and self.value_position is None
-                      and self.q_temp is None and not self.gated)
+                      and self.q_temp is None and not self.gated and not self.whole)
         if self.plain and (s.head_dim % 16 or not 16 <= s.head_dim <= MAX_HEAD_DIM):
             raise ValueError(f"head_dim={s.head_dim} is not supported: the attention kernels take head sizes "
                              f"from 16 to {MAX_HEAD_DIM} in steps of 16")
@@ -85,8 +103,12 @@ class Attention(Mixer):
         }
         if s.cache_from is None:
             wants[f"{prefix}.{n['k']}"] = TensorWant((s.num_kv_heads * s.head_dim, s.hidden_size))
-            wants[f"{prefix}.{n['v']}"] = TensorWant((s.num_kv_heads * self.dv, s.hidden_size))
-        if s.qk_norm_eps is not None and self.norm_weighted:
+            if not self.values_from_keys:
+                wants[f"{prefix}.{n['v']}"] = TensorWant((s.num_kv_heads * self.dv, s.hidden_size))
+        if self.whole:
+            wants[f"{prefix}.{n['q_norm']}"] = TensorWant((s.num_heads * s.head_dim,), "vector")
+            wants[f"{prefix}.{n['k_norm']}"] = TensorWant((s.num_kv_heads * s.head_dim,), "vector")
+        elif s.qk_norm_eps is not None and self.norm_weighted:
             wants[f"{prefix}.{n['q_norm']}"] = TensorWant((s.head_dim,), "vector")
             if s.cache_from is None:
                 wants[f"{prefix}.{n['k_norm']}"] = TensorWant((s.head_dim,), "vector")
@@ -98,7 +120,10 @@ class Attention(Mixer):
         s = self.spec
         n = self._n
         q = tensors[f"{prefix}.{n['q']}"]
-        rows = [q] if s.cache_from is not None else [q, tensors[f"{prefix}.{n['k']}"], tensors[f"{prefix}.{n['v']}"]]
+        if self.values_from_keys:
+            rows = [q, tensors[f"{prefix}.{n['k']}"]]
+        else:
+            rows = [q] if s.cache_from is not None else [q, tensors[f"{prefix}.{n['k']}"], tensors[f"{prefix}.{n['v']}"]]
         if self.gated:  # the gates' rows ride behind q, k and v: one product for all
             rows.append(tensors[f"{prefix}.{n['g']}"])
         self.w_qkv = torch.cat(rows, dim=0) if len(rows) > 1 else q.contiguous()
@@ -113,6 +138,8 @@ class Attention(Mixer):
     def cache_need(self):
         if self.spec.cache_from is not None:
             return None
+        if self.whole:
+            return KVCacheNeed(self.nkv, self.d, self.spec.window, value_dim=self.dv, pooled_block=self.pooled_block)
         if self.plain:
             return KVCacheNeed(self.nkv, self.d, self.spec.window)
         return KVCacheNeed(self.nkv, self.d, self.spec.window, value_dim=self.dv, keep_first=self.keep_first)
@@ -128,8 +155,9 @@ class Attention(Mixer):
         if b is None:
             raise RuntimeError("attention mixer was given no cache")
         owns = s.cache_from is None
-        if self.q_temp is not None or self.gated:
-            raise NotImplementedError("a temperature on the queries and an output gate run in the step program only")
+        if self.q_temp is not None or self.gated or self.whole:
+            raise NotImplementedError("a temperature on the queries, an output gate and the norm over the whole projection run in "
+                                      "the step program only")
         proj = K.linear(h, self.w_qkv)  # [T, (nh + 2 nkv) d] or [T, nh d]
         table = batch.block_table(b.group)
         rope = None if self.position is None else self.position.tables(batch.max_ctx)
@@ -179,10 +207,48 @@ class Attention(Mixer):
         out = self.attend(q, batch, table, b)
         return K.linear(out, self.w_o, as_delta=True)
 
+    # ---- what a pair of mixers asks of each of them (the form normed over the whole projection)
+    @property
+    def w_in(self):
+        return self.w_qkv
+
+    @w_in.setter
+    def w_in(self, value):
+        self.w_qkv = value
+
+    @property
+    def input_cols(self) -> int:
+        return self.nh * self.d + self.nkv * self.d + (0 if self.values_from_keys else self.nkv * self.dv)
+
+    @property
+    def output_cols(self) -> int:
+        return self.nh * self.dv
+
+    def emit_projected(self, program, proj: int, col: int, out: int, out_col: int, out_scale: float, cache) -> None:
+        """The mixer between its two products: the projections lie in the value ``proj`` from column ``col`` on (the rows of
+        ``w_in``), the result goes to the value ``out`` at column ``out_col``, times ``out_scale``."""
+        if not self.whole:
+            raise NotImplementedError("only attention normed over its whole projection reads and writes at columns of wider values")
+        if not isinstance(cache, KVBinding):
+            raise RuntimeError("attention mixer was given no cache")
+        s, b = self.spec, cache
+        k_col = col + self.nh * self.d
+        program.pooled_attention(
+            proj, out, q_col=col, k_col=k_col, v_col=-1 if self.values_from_keys else k_col + self.nkv * self.d, out_col=out_col,
+            q_norm=self.q_norm_w, k_norm=self.k_norm_w, k_cache=b.k_cache, v_cache=b.v_cache, k_pool=b.k_pool, v_pool=b.v_pool,
+            heads=self.nh, kv_heads=self.nkv, head_dim=self.d, value_dim=self.dv, block_size=b.block_size, window=int(s.window),
+            pooled_block=self.pooled_block, group=b.group, eps=float(s.qk_norm_eps), scale=float(s.scale), out_scale=out_scale)
+
     def emit(self, program, h, cache: KVBinding | None = None) -> None:
         s, b = self.spec, cache
         if b is None:
             raise RuntimeError("attention mixer was given no cache")
+        if self.whole:
+            proj = program.linear(h, self.w_qkv)
+            out = program.take(self.output_cols)
+            self.emit_projected(program, proj, 0, out, 0, 1.0, cache)
+            program.linear_delta(out, self.w_o)
+            return
         owns = s.cache_from is None
         qkv = program.linear(h, self.w_qkv)
         out = program.attention(

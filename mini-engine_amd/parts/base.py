@@ -32,7 +32,8 @@ twice has a cache for each run. A mixer states what it needs kept between steps 
 
 * ``KVCacheNeed``: paged keys and values (heads, head size, window; 0 = all keys);
 * ``StateNeed``: a fixed-size tensor per live request (a slot);
-* ``None``: nothing.
+* ``None``: nothing;
+* a pair ``(left need, right need)`` of these, for a mixer made of two mixers: it is given a ``PairBinding``.
 """
 
 from __future__ import annotations
@@ -52,6 +53,8 @@ class KVCacheNeed:
     window: int = 0  # 0: every earlier key stays needed
     value_dim: int | None = None  # size of the value heads (None: head_dim)
     keep_first: int = 0  # with a window: the first keys of a request stay needed as well
+    pooled_block: int = 0  # > 0: beside the pages of tokens, pages of the same shape for the means of blocks of that many keys
+                           # (entry b at page table[b // block_size], slot b % block_size); every page of a request stays needed
 
     @property
     def v_dim(self) -> int:
@@ -72,6 +75,8 @@ class KVBinding:
     k_cache: torch.Tensor  # [pages, kv_heads, block_size, head_dim]
     v_cache: torch.Tensor  # [pages, kv_heads, head_dim, block_size]
     block_size: int
+    k_pool: torch.Tensor | None = None  # pages of pooled blocks, where the need asks for them: the same shapes
+    v_pool: torch.Tensor | None = None
 
 
 @dataclass
@@ -79,6 +84,14 @@ class StateBinding:
     """What a mixer with per-request state is given: one row per slot (the last row is a spare)."""
 
     state: torch.Tensor  # [slots + 1, *shape]
+
+
+@dataclass
+class PairBinding:
+    """What a mixer made of two mixers is given: each one's binding (None for one that keeps nothing)."""
+
+    left: Any
+    right: Any
 
 
 class Part:

@@ -8,7 +8,10 @@
 
     h = norm1(x);  x = x + scale * (mixer(h) + ffn(h))
 
-one norm that both parts read; ``scale`` is the layer spec's ``residual_scale``; the feed-forward may be absent.
+one norm that both parts read; ``scale`` is the layer spec's ``residual_scale``; the feed-forward may be absent. With a
+norm of its own for the feed-forward (both norms of the same x)::
+
+    x = x + scale * (mixer(norm1(x)) + ffn(norm2(x)))
 
 The residual stream ``x`` is kept in float32 and every sum into it is a float32 sum. A block returns
 its feed-forward output unadded; the next norm kernel (of the next block, or the model's final norm)
@@ -73,7 +76,10 @@ class ParallelBlock:
         self.mixer = MIXERS.build(spec.mixer, dtype, device)
         self.ffn = None if spec.ffn is None else FEED_FORWARDS.build(spec.ffn, dtype, device)
         self.mixer_norm = NORMS.build(spec.mixer_norm, dtype, device)
-        self.ffn_norm = None
+        # a norm of its own for the feed-forward, of the same stream (None: both parts read the one norm)
+        self.ffn_norm = None if self.ffn is None or spec.ffn_norm is None else NORMS.build(spec.ffn_norm, dtype, device)
+        if self.ffn_norm is not None and self.ffn_norm.as_fused() is None:
+            raise ValueError("the feed-forward's own norm in a parallel block is RMS-shaped")
         self.scale = float(spec.residual_scale)
 
     def weight_wants(self):
@@ -82,6 +88,8 @@ class ParallelBlock:
         wants.update(self.mixer_norm.weight_wants(s.mixer_norm_name))
         wants.update(self.mixer.weight_wants(s.mixer_prefix))
         if self.ffn is not None:
+            if self.ffn_norm is not None:
+                wants.update(self.ffn_norm.weight_wants(s.ffn_norm_name))
             wants.update(self.ffn.weight_wants(s.ffn_prefix))
         return wants
 
@@ -90,6 +98,8 @@ class ParallelBlock:
         self.mixer_norm.load(tensors, s.mixer_norm_name)
         self.mixer.load(tensors, s.mixer_prefix)
         if self.ffn is not None:
+            if self.ffn_norm is not None:
+                self.ffn_norm.load(tensors, s.ffn_norm_name)
             self.ffn.load(tensors, s.ffn_prefix)
 
     def emit(self, program, cache=None) -> None:
@@ -99,8 +109,13 @@ class ParallelBlock:
             h = program.normed(norm) if norm.as_fused() is not None else program.normed_by(norm)
             h.value()  # the normed activations as a value of their own: two parts read them
             before, program.delta_scale = program.delta_scale, self.scale
+            stays_before = program.delta_stays
             try:
                 for at, (part, extra) in enumerate(parts):
+                    # a second norm reads the stream as the first did: the mixer's result may not add itself into it on the way
+                    program.delta_stays = stays_before or (at == 0 and self.ffn_norm is not None)
+                    if at == 1 and self.ffn_norm is not None:  # the feed-forward's own norm of the same stream
+                        h = program.normed_again(self.ffn_norm)
                     if callable(getattr(part, "emit", None)):
                         out = part.emit(program, h, *extra)
                     else:
@@ -111,6 +126,7 @@ class ParallelBlock:
                         program.hold()  # set aside: the next norm's kernel adds it together with the last part's result
             finally:
                 program.delta_scale = before
+                program.delta_stays = stays_before
 
 
 class HyperConnectionBlock:

@@ -7,6 +7,10 @@ ff]``); the router's weight is kept in float32. A step routes on the device: the
 expert and served in tiles of one expert (``csrc/routed_ff.hip``), so a decode step reads the weights of the experts
 that its tokens picked and no others. The results wait as float32 partial sums, one per pick of a token, that the
 next add of the residual stream sums up in the order of the picks.
+
+The spec may also: score by the sigmoid of the logits and weight the picks by their scores over their sum, times a scale;
+bound the picks to the experts of the best few of some equal groups of neighbours; give the activation a limit to clamp by;
+and add an expert that every token uses, multiplied by the sigmoid of one number per token (one more partial sum).
 """
 
 from __future__ import annotations
@@ -23,14 +27,24 @@ class RoutedExperts(FeedForward):
 
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
-        if spec.activation not in K.GATE_ACTIVATIONS:
-            raise ValueError(f"routed experts know the activations {sorted(K.GATE_ACTIVATIONS)}, got {spec.activation!r}")
+        known = sorted(set(K.GATE_ACTIVATIONS) | set(K.LIMITED_GATE_ACTIVATIONS))
+        if spec.activation not in known:
+            raise ValueError(f"routed experts know the activations {known}, got {spec.activation!r}")
         if not 1 <= spec.top_k <= spec.num_experts:
             raise ValueError(f"{spec.top_k} of {spec.num_experts} experts a token")
+        self.scoring = getattr(spec, "scoring", "softmax_picked")
+        self.groups, self.keep = int(getattr(spec, "num_groups", 1)), int(getattr(spec, "keep_groups", 1))
+        if self.scoring == "softmax_picked" and (self.groups, self.keep) != (1, 1):
+            raise ValueError("groups of experts bound the picks of a router that scores by sigmoid_normalized")
+        if (self.groups < 1 or spec.num_experts % self.groups or not 1 <= self.keep <= self.groups
+                or self.keep * (spec.num_experts // self.groups) < spec.top_k):
+            raise ValueError(f"{spec.num_experts} experts in {self.groups} groups of which {self.keep} are kept, {spec.top_k} picks")
+        self.shared_size = int(getattr(spec, "shared_size", 0))
         names = dict(getattr(spec, "names", ()) or ())
         self._n = {r: names.get(r, d) for r, d in (("router", "router"), ("expert", "experts."), ("gate", "gate_proj.weight"),
-                                                    ("up", "up_proj.weight"), ("down", "down_proj.weight"))}
-        self.router = self.w_gate_up = self.w_down = None
+                                                    ("up", "up_proj.weight"), ("down", "down_proj.weight"), ("shared", "shared"),
+                                                    ("shared_gate", "gate"))}
+        self.router = self.w_gate_up = self.w_down = self.w_shared_gate_up = self.w_shared_down = None
 
     def _expert(self, prefix: str, e: int, role: str) -> str:
         return f"{prefix}.{self._n['expert']}{e}.{self._n[role]}"
@@ -42,6 +56,12 @@ class RoutedExperts(FeedForward):
             wants[self._expert(prefix, e, "gate")] = TensorWant((s.intermediate_size, s.hidden_size))
             wants[self._expert(prefix, e, "up")] = TensorWant((s.intermediate_size, s.hidden_size))
             wants[self._expert(prefix, e, "down")] = TensorWant((s.hidden_size, s.intermediate_size))
+        if self.shared_size:
+            sp = f"{prefix}.{self._n['shared']}"
+            wants[f"{sp}.{self._n['gate']}"] = TensorWant((self.shared_size, s.hidden_size))
+            wants[f"{sp}.{self._n['up']}"] = TensorWant((self.shared_size, s.hidden_size))
+            wants[f"{sp}.{self._n['down']}"] = TensorWant((s.hidden_size, self.shared_size))
+            wants[f"{sp}.{self._n['shared_gate']}"] = TensorWant((1, s.hidden_size), "vector")
         return wants
 
     def load(self, tensors, prefix: str) -> None:
@@ -50,14 +70,24 @@ class RoutedExperts(FeedForward):
         self.w_gate_up = torch.stack([torch.cat((tensors[self._expert(prefix, e, "gate")], tensors[self._expert(prefix, e, "up")]), dim=0)
                                       for e in range(s.num_experts)]).contiguous()
         self.w_down = torch.stack([tensors[self._expert(prefix, e, "down")] for e in range(s.num_experts)]).contiguous()
+        if self.shared_size:
+            sp = f"{prefix}.{self._n['shared']}"
+            self.w_shared_gate_up = torch.cat((tensors[f"{sp}.{self._n['gate']}"], tensors[f"{sp}.{self._n['up']}"]), dim=0)
+            self.w_shared_down = tensors[f"{sp}.{self._n['down']}"]
+            # the shared expert's gate as one more row of the router: the kernel that routes a token computes it on the way
+            self.router = torch.cat((self.router, tensors[f"{sp}.{self._n['shared_gate']}"].reshape(1, -1)), dim=0).contiguous()
 
     def forward(self, h, batch=None):
         raise NotImplementedError("routed experts run in the step program only")
 
     def emit(self, program, h) -> None:
         x = h.value() if hasattr(h, "value") else h
-        program.routed_ff(x, router=self.router, gate_up=self.w_gate_up, down=self.w_down, top_k=int(self.spec.top_k),
-                          activation=self.spec.activation)
+        s = self.spec
+        program.routed_ff(x, router=self.router, gate_up=self.w_gate_up, down=self.w_down, top_k=int(s.top_k), activation=s.activation,
+                          activation_limit=float(getattr(s, "activation_limit", 0.0)), scoring=self.scoring, num_groups=self.groups,
+                          keep_groups=self.keep, route_scale=float(getattr(s, "route_scale", 1.0)),
+                          shared_gate_up=self.w_shared_gate_up, shared_down=self.w_shared_down,
+                          shared_limit=float(getattr(s, "shared_limit", 0.0)))
 
 
 FEED_FORWARDS.register("routed_experts", RoutedExperts)
