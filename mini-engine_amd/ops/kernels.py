@@ -1361,3 +1361,122 @@ def gemm_bf16_stream_norm_streams(xs: torch.Tensor, delta, rewrite: torch.Tensor
         _i64(m * k), _p(rewrite), _p(reads), _p(norm_weight), _f(eps), _p(new if pending else None), _p(weight), _p(out), _i(m), _i(n),
         _i(k), _i(gate), _i(_code(out_dtype)), _i(compute_units(xs.device)), _stream()))
     return out, new
+
+
+# ------------------------------------------------------------------ attention over a window and pooled blocks
+def whole_norm_scatter(proj: torch.Tensor, q_w: torch.Tensor, k_w: torch.Tensor, positions, token_item, block_table, k_cache, v_cache,
+                       nh: int, nkv: int, d: int, dv: int, eps: float, q_col: int = 0, k_col: int | None = None, v_col: int = -1,
+                       k_pool: torch.Tensor | None = None, v_pool: torch.Tensor | None = None, pooled_block: int = 0) -> torch.Tensor:
+    """q and k of ``proj`` ``[T, row]`` (queries at column ``q_col``, keys at ``k_col``, default right behind the queries) normed over
+    their whole projection with the float32 weights ``q_w`` ``[nh * d]`` and ``k_w`` ``[nkv * d]``; the normed keys go to the key pages,
+    the values (the column ``v_col``; -1: the keys as projected) to the value pages; with ``pooled_block`` P the means of the blocks
+    of P keys and values that the step's tokens complete go to the pooled pages. Returns the normed queries ``[T, nh, d]``."""
+    _want(proj, "proj", None, (None, None))
+    t, row = proj.shape
+    k_col = q_col + nh * d if k_col is None else k_col
+    _want(q_w, "q_w", torch.float32, (nh * d,))
+    _want(k_w, "k_w", torch.float32, (nkv * d,))
+    bs = k_cache.shape[2]
+    _check_cache(k_cache, v_cache, proj.dtype, nkv, d, bs, dv)
+    _check_step_index(positions, token_item, block_table, t)
+    if pooled_block:
+        _want(k_pool, "k_pool", proj.dtype, tuple(k_cache.shape))
+        _want(v_pool, "v_pool", proj.dtype, tuple(v_cache.shape))
+    q = torch.empty((t, nh, d), dtype=proj.dtype, device=proj.device)
+    check(lib().me_whole_norm_scatter(_p(proj), _i64(row), _i(q_col), _i(k_col), _i(v_col), _p(q_w), _p(k_w), _p(positions), _p(token_item),
+                                      _p(block_table), _i(block_table.shape[1]), _p(q), _p(k_cache), _p(v_cache), _p(k_pool), _p(v_pool),
+                                      _i(t), _i(nh), _i(nkv), _i(d), _i(dv), _i(bs), _i(pooled_block), _f(eps), _i(_code(proj.dtype)),
+                                      _stream()))
+    return q
+
+
+def attention_pooled(q, k_cache, v_cache, k_pool, v_pool, positions, token_item, block_table, scale: float, window: int,
+                     pooled_block: int, out: torch.Tensor | None = None, out_col: int = 0, out_scale: float = 1.0) -> torch.Tensor:
+    """Causal attention of q ``[T, nh, d]`` over the window's keys and, with ``pooled_block`` P, the pooled entries of the whole
+    blocks of P positions before the window (one softmax for both). The result, times ``out_scale``, goes to ``out`` (default:
+    a new ``[T, nh * dv]``) at column ``out_col``."""
+    _want(q, "q", None, (None, None, None))
+    t, nh, d = q.shape
+    nkv, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
+    _check_cache(k_cache, v_cache, q.dtype, nkv, d, bs, dv)
+    _check_step_index(positions, token_item, block_table, t)
+    if pooled_block:
+        _want(k_pool, "k_pool", q.dtype, tuple(k_cache.shape))
+        _want(v_pool, "v_pool", q.dtype, tuple(v_cache.shape))
+    if out is None:
+        out = torch.empty((t, nh * dv), dtype=q.dtype, device=q.device)
+    _want(out, "out", q.dtype, (t, None))
+    if out_col < 0 or out_col + nh * dv > out.shape[1]:
+        raise ValueError(f"the result at column {out_col} of rows of {out.shape[1]}")
+    check(lib().me_attention_general_pooled(
+        _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(token_item), _p(block_table), _i(block_table.shape[1]), _p(out), _i(t),
+        _i(nh), _i(nkv), _i(d), _i(dv), _i(bs), _i(window), _i(0), _p(None), _i(0), _f(scale), _p(None), _p(None), _i64(0),
+        _p(k_pool), _p(v_pool), _i(pooled_block), _i64(out.shape[1]), _i(out_col), _f(out_scale), _i(_code(q.dtype)),
+        _i(block_table.shape[0]), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ the generalized delta rule
+def delta_rule(proj: torch.Tensor, cols: dict, w2: torch.Tensor, w0: torch.Tensor, a_bias: torch.Tensor, norm_w: torch.Tensor,
+               state: torch.Tensor, item_start: torch.Tensor, state_slots: torch.Tensor, heads: int, d: int, eps: float,
+               decay_coef: float, out: torch.Tensor | None = None, out_col: int = 0, out_scale: float = 1.0) -> torch.Tensor:
+    """Linear attention by the generalized delta rule over the items of a step (``item_start`` int32 ``[items + 1]``, ``state_slots``
+    int32 ``[items]``), from and into their rows of ``state`` float32 ``[slots, heads, d, d]``. ``proj`` ``[T, row]`` holds r, k, v, the
+    gate ``g`` and the removal rate ``a`` (``heads * d`` columns each) and the decay's inner projection ``w1`` at the columns that
+    ``cols`` names; ``w2`` ``[heads * d, rank]`` in the activations' type; ``w0``, ``a_bias``, ``norm_w`` float32 ``[heads * d]``. The
+    normed, gated result, times ``out_scale``, goes to ``out`` (default: a new ``[T, heads * d]``) at column ``out_col``."""
+    _want(proj, "proj", None, (None, None))
+    t, row = proj.shape
+    n = heads * d
+    _want(w2, "w2", proj.dtype, (n, None))
+    rank = w2.shape[1]
+    for name, v in (("w0", w0), ("a_bias", a_bias), ("norm_w", norm_w)):
+        _want(v, name, torch.float32, (n,))
+    _want(state, "state", torch.float32, (None, heads, d, d))
+    items = state_slots.shape[0]
+    _want(item_start, "item_start", torch.int32, (items + 1,))
+    _want(state_slots, "state_slots", torch.int32, (items,))
+    if out is None:
+        out = torch.empty((t, n), dtype=proj.dtype, device=proj.device)
+    _want(out, "out", proj.dtype, (t, None))
+    check(lib().me_delta_rule(_p(proj), _i64(row), _i(cols["r"]), _i(cols["k"]), _i(cols["v"]), _i(cols["g"]), _i(cols["a"]), _i(cols["w1"]),
+                              _p(w2), _p(w0), _p(a_bias), _p(norm_w), _p(state), _p(item_start), _p(state_slots), _p(out),
+                              _i64(out.shape[1]), _i(out_col), _f(out_scale), _i(t), _i(items), _i(heads), _i(d), _i(rank), _f(eps),
+                              _f(decay_coef), _i(_code(proj.dtype)), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ routed experts that score by sigmoid
+def routed_ff_scored(h: torch.Tensor, router: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, top_k: int, activation: str,
+                     limit: float, scoring: str, num_groups: int, keep_groups: int, route_scale: float, shared: bool = False):
+    """As :func:`routed_ff`, with the activation's ``limit``, the way of ``scoring`` ("softmax_picked", "sigmoid_normalized"), the
+    picks bounded to the ``keep_groups`` best of ``num_groups`` groups and the weights times ``route_scale``. ``shared``: the
+    router has one more row behind the experts'; the sigmoid of every token's product with it is returned as well (float32 ``[T]``)."""
+    t, hidden = h.shape
+    e, two_ff, _ = gate_up.shape
+    _want(router, "router", torch.float32, (e + (1 if shared else 0), hidden))
+    _want(gate_up, "gate_up", h.dtype, (e, two_ff, hidden))
+    _want(down, "down", h.dtype, (e, hidden, two_ff // 2))
+    lib().me_routed_ff_workspace.restype = ctypes.c_longlong
+    need = lib().me_routed_ff_workspace(_i64(t), _i(e), _i(top_k), _i(two_ff // 2), _i(h.element_size()))
+    ws = torch.empty(int(need), dtype=torch.uint8, device=h.device)
+    parts = torch.empty((top_k, t, hidden), dtype=torch.float32, device=h.device)
+    gate = torch.empty(t, dtype=torch.float32, device=h.device) if shared else None
+    codes = {"softmax_picked": 0, "sigmoid_normalized": 1}
+    check(lib().me_routed_ff_scored(_p(h), _p(router), _p(gate_up), _p(down), _p(parts), _p(ws), _i(t), _i(hidden), _i(e), _i(top_k),
+                                    _i(two_ff // 2), _i(gate_code(activation, limited=True)), _f(limit), _i(codes[scoring]),
+                                    _i(num_groups), _i(keep_groups), _f(route_scale), _p(gate), _i(_code(h.dtype)), _stream()))
+    return (PartialSums(parts), gate) if shared else PartialSums(parts)
+
+
+def gated_rows(gate_up: torch.Tensor, row_gate: torch.Tensor | None, activation: str, limit: float = 0.0) -> torch.Tensor:
+    """``act(gate_up[:, :I], gate_up[:, I:])`` for gate_up ``[T, 2I]`` by any activation, those with a limit among them, every row
+    times ``row_gate`` (float32 ``[T]`` or None)."""
+    _want(gate_up, "gate_up", None, (None, None))
+    t, two_i = gate_up.shape
+    if row_gate is not None:
+        _want(row_gate, "row_gate", torch.float32, (t,))
+    out = torch.empty((t, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+    check(lib().me_gated_rows(_p(gate_up), _p(row_gate), _p(out), _i(t), _i(two_i // 2), _i(gate_code(activation, limited=True)), _f(limit),
+                              _i(_code(gate_up.dtype)), _stream()))
+    return out

@@ -99,8 +99,9 @@ def clamped_expert(h, w, prefix: str, limit: float):
     return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ w[prefix + ".down"].T
 
 
-def route(z, r: dict):
-    """Router logits z [T, E] -> (picked experts [T, top], their weights [T, top])."""
+def route(z, r: dict, gaps: list | None = None):
+    """Router logits z [T, E] -> (picked experts [T, top], their weights [T, top]). ``gaps`` collects, per token, how far the
+    closest decision was from going the other way (between the last group kept and the next, the last pick and the next)."""
     experts, top = int(r["experts"]), int(r["top"])
     count, keep = int(r["groups"]["count"]), int(r["groups"]["keep"])
     s = torch.sigmoid(z)
@@ -112,15 +113,25 @@ def route(z, r: dict):
     allowed = torch.zeros(t, count, dtype=torch.bool)
     allowed.scatter_(1, best, True)
     allowed = allowed.unsqueeze(-1).expand(t, count, per).reshape(t, experts)
-    picked = s.masked_fill(~allowed, -math.inf).topk(top, dim=-1).indices
+    masked = s.masked_fill(~allowed, -math.inf)
+    picked = masked.topk(top, dim=-1).indices
+    if gaps is not None:
+        gap = torch.full((t,), math.inf, dtype=s.dtype)
+        if keep < count:
+            ordered = group_score.sort(dim=-1, descending=True).values
+            gap = torch.minimum(gap, ordered[:, keep - 1] - ordered[:, keep])
+        if top < keep * per:
+            ordered = masked.sort(dim=-1, descending=True).values
+            gap = torch.minimum(gap, ordered[:, top - 1] - ordered[:, top])
+        gaps.append(gap)
     weights = s.gather(1, picked)
     weights = weights / (weights.sum(dim=-1, keepdim=True) + 1e-20) * float(r["scale"])
     return picked, weights
 
 
-def routed_experts(h, w, prefix: str, mlp: dict):
+def routed_experts(h, w, prefix: str, mlp: dict, gaps: list | None = None):
     r = mlp["router"]
-    picked, weights = route(h @ w[prefix + ".router"].T, r)
+    picked, weights = route(h @ w[prefix + ".router"].T, r, gaps)
     limit = float(mlp["expert"]["limit"])
     out = torch.zeros_like(h)
     for e in range(int(r["experts"])):
@@ -133,8 +144,10 @@ def routed_experts(h, w, prefix: str, mlp: dict):
     return out
 
 
-def forward(cfg: dict, w: dict, tokens, want=None, residuals: list | None = None):
-    """Logits [wanted or all, vocab] of one sequence from position 0; ``residuals`` collects the stream after every layer."""
+def forward(cfg: dict, w: dict, tokens, want=None, residuals: list | None = None, router_gaps: list | None = None, after_norm=None):
+    """Logits [wanted or all, vocab] of one sequence from position 0; ``residuals`` collects the stream after every layer,
+    ``router_gaps`` every router's closest decision per token; ``after_norm`` is applied to every part's normed input."""
+    after_norm = after_norm or (lambda z: z)
     w = {name: t.to(F64) for name, t in w.items()}
     eps, groups = float(cfg["norm"]["eps"]), int(cfg["norm"]["groups"])
     x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)]
@@ -142,13 +155,13 @@ def forward(cfg: dict, w: dict, tokens, want=None, residuals: list | None = None
         p = f"l{int(layer.get('weights_of', i))}"
         if layer["type"] != "parallel":
             raise ValueError(layer["type"])
-        delta = pair_mixer(group_rms_norm(x, w[p + ".norm1"], groups, eps), w, p + ".mix", layer["mixer"], eps)
+        delta = pair_mixer(after_norm(group_rms_norm(x, w[p + ".norm1"], groups, eps)), w, p + ".mix", layer["mixer"], eps)
         if layer.get("mlp") is not None:
-            delta = delta + routed_experts(group_rms_norm(x, w[p + ".norm2"], groups, eps), w, p + ".mlp", layer["mlp"])
+            delta = delta + routed_experts(after_norm(group_rms_norm(x, w[p + ".norm2"], groups, eps)), w, p + ".mlp", layer["mlp"], router_gaps)
         x = x + delta
         if residuals is not None:
             residuals.append(x.clone())
     if want is not None:
         x = x[torch.as_tensor(want, dtype=torch.long)]
-    x = group_rms_norm(x, w["final.norm"], groups, eps)
+    x = after_norm(group_rms_norm(x, w["final.norm"], groups, eps))
     return (x @ w["embed"].T) * float(cfg["logit_scale"])
