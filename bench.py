@@ -388,16 +388,39 @@ def kifezen_config(size: str):
                                     "norm": {"eps": 1e-6}, "layers": order})
 
 
-DESIGNS = {"gonurax": ("Gonurax", gonurax_config), "kifezen": ("Kifezen", kifezen_config)}
+def bezurax_config(size: str):
+    """Eight parallel layers, each a pair of mixers and routed experts. Left: 16 heads of 128 on 8 key/value heads whose values
+    are the keys, a window of 1,024 keys beside the means of blocks of 32. Right: the generalized delta rule over heads of 64
+    (as many as fill the width), a decay of inner size 64. Feed-forward: 16 experts of a third of the size's feed-forward, two a
+    token out of the best two of four groups, and a shared expert of the same size (as many weights at work per token as in
+    the dense feed-forward of the models beside it). Four layers have weights of their own, the other four run theirs again."""
+    from mini_engine_amd.models.bezurax import BezuraxConfig
+
+    z = DESIGN_SIZES[size]
+    ff = z["ff"] // 3
+    left = {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024, "pool": 32}}
+    right = {"heads": z["width"] // 64, "dim": 64, "decay_rank": 64}
+    mlp = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "shared": {"ff": ff, "limit": 7.0},
+           "router": {"experts": 16, "top": 2, "groups": {"count": 4, "keep": 2}, "scale": 2.5}}
+    layer = {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}, "mlp": mlp}
+    order = [dict(layer) for _ in range(DESIGN_LAYERS // 2)] + [dict(layer, weights_of=i) for i in range(DESIGN_LAYERS // 2)]
+    return BezuraxConfig.from_dict({"architecture": "Bezurax", "vocab": DESIGN_VOCAB, "width": z["width"], "logit_scale": 1.0,
+                                    "norm": {"eps": 1e-6, "groups": 2}, "layers": order})
+
+
+# design -> (architecture, its configuration at a size, the model beside it: "qwen3" or another design of this table)
+DESIGNS = {"gonurax": ("Gonurax", gonurax_config, "qwen3"), "kifezen": ("Kifezen", kifezen_config, "qwen3"),
+           "bezurax": ("Bezurax", bezurax_config, "gonurax")}
 
 
 def design_line(args) -> dict:
-    """Prefill and decode throughput of a design (Gonurax, Kifezen) beside the Qwen3 dense design at equal layer sizes (random
+    """Prefill and decode throughput of a design beside the model closest to it (the Qwen3 dense design for Gonurax and Kifezen,
+    the Gonurax design, which has windowed attention beside recurrent layers, for Bezurax) at equal layer sizes (random
     weights, eight layers): a 2,048-token prompt, and decode steps at batch 1, 8 and 64 behind a context of 2,304."""
     from mini_engine_amd.models.qwen3 import Qwen3Config
 
     design = args.design
-    arch_name, config_of = DESIGNS[design]
+    arch_name, config_of, beside = DESIGNS[design]
     batches = [int(b) for b in args.design_batches.split(",") if b]
     headline = 8 if 8 in batches else batches[0]
     ctx, out = 2304, {}
@@ -407,8 +430,9 @@ def design_line(args) -> dict:
         qwen = Qwen3Config(vocab_size=DESIGN_VOCAB, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, num_hidden_layers=DESIGN_LAYERS,
                            hidden_size=z["width"], num_attention_heads=z["heads"], num_key_value_heads=8,
                            intermediate_size=z["ff"], tie_word_embeddings=True, max_position_embeddings=40960)
-        for name, arch, cfg in ((design, arch_name, config_of(size)), ("qwen3", "Qwen3ForCausalLM", qwen)):
-            if args.design_alone and name == "qwen3":
+        other = ("qwen3", "Qwen3ForCausalLM", qwen) if beside == "qwen3" else (beside, DESIGNS[beside][0], DESIGNS[beside][1](size))
+        for name, arch, cfg in ((design, arch_name, config_of(size)), other):
+            if args.design_alone and name == beside:
                 continue
             bench = DecodeBench(cfg, args.dtype, ctx, max(batches), architecture=arch)
             pf = bench.prefill(args.prefill_tokens)
@@ -427,7 +451,7 @@ def design_line(args) -> dict:
             "warmup": args.warmup, "ms_per_step": out[f"{design}_{first}_decode_b{headline}_ms_per_step"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic: seeded uniform-random token ids, random N(0, 0.02) weights",
-            "config": {"model": f"{arch_name} design beside the Qwen3 dense design at equal layer sizes", "layers": DESIGN_LAYERS,
+            "config": {"model": f"{arch_name} design beside the {'Qwen3 dense' if beside == 'qwen3' else DESIGNS[beside][0]} design at equal layer sizes", "layers": DESIGN_LAYERS,
                        "vocab": DESIGN_VOCAB, "sizes": {z: DESIGN_SIZES[z] for z in sizes}, "seq_len": ctx, "global_batch": headline,
                        "parallelism": "single GPU"},
             "points": out}
@@ -447,11 +471,11 @@ def main() -> int:
     ap.add_argument("--skip-prefill", action="store_true", help="profiling aid: do not measure the prefill")
     ap.add_argument("--skip-extras", action="store_true",
                     help="profiling aid: only the decode steps and the prefill (no serving workloads, no float32 point, no probes)")
-    ap.add_argument("--design", default="", choices=["", "gonurax", "kifezen"],
-                    help="instead of the default workload: this design beside the Qwen3 dense design at equal layer sizes")
+    ap.add_argument("--design", default="", choices=["", "gonurax", "kifezen", "bezurax"],
+                    help="instead of the default workload: this design beside the model closest to it at equal layer sizes")
     ap.add_argument("--design-sizes", default="1024,2048", help="widths of --design to measure, comma separated")
     ap.add_argument("--design-batches", default="1,8,64", help="decode batch sizes of --design, comma separated")
-    ap.add_argument("--design-alone", action="store_true", help="profiling aid: --design without the Qwen3 model beside it")
+    ap.add_argument("--design-alone", action="store_true", help="profiling aid: --design without the model beside it")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on one GPU)")
