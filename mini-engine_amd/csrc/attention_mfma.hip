@@ -170,6 +170,16 @@ struct DecodeFusedArgs {
   // (for every launch, fused or not) with a window: the first keys of an item that stay visible behind it. Their tiles
   // come before the window's in the order in which an item's tiles are dealt to the splits.
   int keep_first = 0;
+  // (unfused launches) with a window and pool_block P > 0: pages of pooled entries, entry b the mean of the keys (and of the
+  // values) at the positions b P .. b P + P - 1, at page table[b / bs], slot b % bs. An item sees the entries of the blocks that
+  // its window has wholly left behind, beside the window's keys. Their tiles stand before the window's, as kept first keys' do.
+  const bf16_t* k_pool = nullptr;
+  const bf16_t* v_pool = nullptr;
+  int pool_block = 0;
+  // where the finished output goes: rows out_row elements apart (0: nh * D), from column out_col on, times out_scale
+  long long out_row = 0;
+  int out_col = 0;
+  float out_scale = 1.f;
 };
 
 // Tiles of a split from which on a wave fetches one tile at a time, whatever DEPTH says: with five tiles and more of its own
@@ -202,12 +212,11 @@ __device__ __forceinline__ void attention_decode_body(
   const int heads_here = min(16, group - chunk * 16);
   const int head0 = kvh * group + chunk * 16;
   const int* table = block_table + (size_t)item * table_width;
-  auto fetch = [&](KvTile<D>& t, int key0) {
+  auto fetch_from = [&](KvTile<D>& t, int key0, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc) {
     int page = table[min(key0 >> bs_shift, table_width - 1)];
     page = page < 0 ? 0 : page;
     const int off = key0 & (bs - 1);
-    load_tile<D, STREAMED>(t, k_cache + (((size_t)page * nkv + kvh) * bs + off) * D,
-                           v_cache + ((size_t)page * nkv + kvh) * D * bs + off, bs);
+    load_tile<D, STREAMED>(t, kc + (((size_t)page * nkv + kvh) * bs + off) * D, vc + ((size_t)page * nkv + kvh) * D * bs + off, bs);
   };
   KvTile<D> t[DEPTH];
   // The keys of an item, from its window's first (rounded down to a tile of 16) to its newest, are dealt
@@ -227,9 +236,19 @@ __device__ __forceinline__ void attention_decode_body(
   // Kept first keys that the window has left behind: their tiles (keys 0 .. kept16 - 1) stand before the window's, at the
   // places vlo .. lo16 - 1 of the run of tiles that is dealt to the splits; `key_at` gives a place's key.
   const int keep_first = fa.keep_first;
-  const int kept16 = keep_first > 0 && lo16 > 0 ? min((keep_first + 15) / 16 * 16, lo16) : 0;
+  // Pooled entries that the item sees (those of the blocks before its window): their tiles (entries 0 .. pooled16 - 1) stand
+  // at those places instead; places may then begin below zero.
+  const int pool_block = fa.pool_block;
+  const int pooled = pool_block > 0 ? lo / pool_block : 0;
+  const int kept16 = pool_block > 0 ? (pooled + 15) / 16 * 16 : keep_first > 0 && lo16 > 0 ? min((keep_first + 15) / 16 * 16, lo16) : 0;
   const int vlo = lo16 - kept16;
   auto key_at = [&](int place) { return place < lo16 ? place - vlo : place; };
+  auto fetch = [&](KvTile<D>& t, int place) {
+    if (pool_block > 0 && place < lo16)
+      fetch_from(t, place - vlo, fa.k_pool, fa.v_pool);
+    else
+      fetch_from(t, key_at(place), k_cache, v_cache);
+  };
   int tiles_per_split = ((ctx - vlo + 15) / 16 + splits - 1) / splits;
   // With 16 splits and more per item, runs of 16, 32, 48 or 64 tiles (the waves of an item then start at keys a multiple of 256
   // apart and walk them in step) measured slower than runs one tile longer with a split less at work, on the same GPU in turns:
@@ -253,7 +272,7 @@ __device__ __forceinline__ void attention_decode_body(
     // the first tile is requested before the query is prepared, unless it holds the slot that this
     // block is about to write
     const bool early = !FUSED || begin + 16 < ctx;
-    if (early) fetch(t[0], key_at(begin));
+    if (early) fetch(t[0], begin);
     Frag8 qf[1][D / 32];
     if (FUSED) {
       constexpr int HC = D / 64;  // chunks per half head
@@ -349,8 +368,15 @@ __device__ __forceinline__ void attention_decode_body(
           qf[0][c].u = *reinterpret_cast<const uint4*>(q + ((size_t)item * nh + head0 + r) * D + c * 32 + g * 8);
       }
     }
-    const int qpos[1] = {ctx - 1};
-    if (!early) fetch(t[0], key_at(begin));
+    // the tile at a place: a pooled tile shows its entries below `pooled`, any other the keys from `lo` (or kept) to the newest
+    auto run_tile = [&](const KvTile<D>& tile, int place) {
+      const bool of_pool = pool_block > 0 && place < lo16;
+      const int key0 = key_at(place);
+      const int qpos[1] = {of_pool ? pooled - 1 : ctx - 1};
+      compute_tile<D, 1>(tile, key0, of_pool ? 0 : lo, qpos, of_pool ? key0 + 16 > pooled : (place < lo || place + 16 > ctx), qf,
+                         scale_log2, m, lsum, acc, of_pool ? 0 : keep_first);
+    };
+    if (!early) fetch(t[0], begin);
     // DEPTH tiles in flight per wave: tile i + DEPTH - 1 is requested before the products of tile i. Short
     // splits (few waves, each waiting on memory) want two (four measured no better); with long splits the
     // chip is full of waves and fewer registers, one more wave per SIMD, serve better. A tile past `end` is a valid page that
@@ -358,20 +384,20 @@ __device__ __forceinline__ void attention_decode_body(
     if (DEPTH > 1 && tiles_per_split > LONG_RUN) {
       // a long run of this wave's own (the chip is full of such waves): one tile at a time streams best
       for (int k = begin; k < end; k += 16) {
-        if (k > begin) fetch(t[0], key_at(k));
-        compute_tile<D, 1>(t[0], key_at(k), lo, qpos, k < lo || k + 16 > ctx, qf, scale_log2, m, lsum, acc, keep_first);
+        if (k > begin) fetch(t[0], k);
+        run_tile(t[0], k);
       }
     } else {
 #pragma unroll
-      for (int j = 1; j < DEPTH - 1; ++j) fetch(t[j], key_at(begin + 16 * j));
+      for (int j = 1; j < DEPTH - 1; ++j) fetch(t[j], begin + 16 * j);
       for (int key0 = begin; key0 < end; key0 += 16 * DEPTH) {
 #pragma unroll
         for (int j = 0; j < DEPTH; ++j) {
           const int k = key0 + 16 * j;
-          if (DEPTH > 1) fetch(t[(j + DEPTH - 1) % DEPTH], key_at(k + 16 * (DEPTH - 1)));
-          else if (k > begin) fetch(t[0], key_at(k));
+          if (DEPTH > 1) fetch(t[(j + DEPTH - 1) % DEPTH], k + 16 * (DEPTH - 1));
+          else if (k > begin) fetch(t[0], k);
           if (j == 0 || k < end)
-            compute_tile<D, 1>(t[j], key_at(k), lo, qpos, k < lo || k + 16 > ctx, qf, scale_log2, m, lsum, acc, keep_first);
+            run_tile(t[j], k);
         }
       }
     }
@@ -432,8 +458,9 @@ __device__ __forceinline__ void attention_decode_body(
         denom = denom * keep + fast_exp2(s2 - top);
         total[0] *= keep, total[1] *= keep, total[2] *= keep, total[3] *= keep;
       }
-      const float inv = denom > 0.f ? 1.f / denom : 0.f;  // no visible key at all: zeros, not NaN
-      *reinterpret_cast<short4_t*>(out + head * D + quad * 4) =
+      const float inv = denom > 0.f ? fa.out_scale / denom : 0.f;  // no visible key at all: zeros, not NaN
+      bf16_t* orow = fa.out_row > 0 ? out + (size_t)item * fa.out_row + fa.out_col + (size_t)(head0 + hr) * D : out + head * D;
+      *reinterpret_cast<short4_t*>(orow + quad * 4) =
           pack_bf16x4(total[0] * inv, total[1] * inv, total[2] * inv, total[3] * inv);
     } else {
       const size_t slot = head * blocks_z + blockIdx.z;
@@ -478,7 +505,8 @@ __global__ __launch_bounds__(DECODE_BLOCK_WAVES(D) * 64) void attention_decode_k
 __global__ __launch_bounds__(256) void attention_decode_combine_kernel(const float* __restrict__ part_o,
                                                                        const float* __restrict__ part_ml,
                                                                        bf16_t* __restrict__ out, int num_splits, int d,
-                                                                       const float* __restrict__ sink, int nh) {
+                                                                       const float* __restrict__ sink, int nh, long long out_row,
+                                                                       int out_col, float out_scale) {
   __shared__ float wgt[ME_MAX_SPLITS];
   __shared__ float red_max[4], red_sum[4];
   __shared__ float4_t partial[256];
@@ -551,8 +579,9 @@ __global__ __launch_bounds__(256) void attention_decode_combine_kernel(const flo
       total[2] += v[2];
       total[3] += v[3];
     }
-    const float inv = 1.f / denom;
-    *reinterpret_cast<short4_t*>(out + unit * d + tid * 4) =
+    const float inv = out_scale / denom;
+    bf16_t* orow = out_row > 0 ? out + (unit / nh) * out_row + out_col + (unit % nh) * d : out + unit * d;
+    *reinterpret_cast<short4_t*>(orow + tid * 4) =
         pack_bf16x4(total[0] * inv, total[1] * inv, total[2] * inv, total[3] * inv);
   }
 }
@@ -562,8 +591,10 @@ static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, c
                           int width, float* part_o, float* part_ml, int items, int nh, int nkv, int bs, int window,
                           float scale_log2, int depth, int num_splits, int block_waves, bf16_t* out,
                           const DecodeFusedArgs* fused, const int* live_items, int waves_wanted, int streamed,
-                          const int* step_flags, int keep_first, const float* sink, hipStream_t stream) {
+                          const int* step_flags, int keep_first, const float* sink, const DecodeFusedArgs* pool,
+                          hipStream_t stream) {
   DecodeFusedArgs unfused{};
+  if (pool) unfused = *pool;
   unfused.keep_first = keep_first;
   const int chunks = (nh / nkv + 15) / 16;
   dim3 grid(items, nkv * chunks, num_splits / block_waves);  // num_splits is a multiple of block_waves
@@ -657,7 +688,7 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
                          int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
                          int max_ctx, const DecodeFusedArgs* fused, const int* live_items, int full_splits,
                          int waves_wanted, const int* step_flags, hipStream_t stream, int keep_first = 0,
-                         const float* sink = nullptr);
+                         const float* sink = nullptr, const DecodeFusedArgs* pool = nullptr);
 
 // As me_attention_decode_bf16, with the first `keep_first` keys of every item visible behind the window.
 extern "C" int me_attention_decode_bf16_kept(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
@@ -673,6 +704,27 @@ extern "C" int me_attention_decode_bf16_kept(const void* q, const void* k_cache,
 
 // As me_attention_decode_bf16, with a learned logit per head (sink float32 [nh], not multiplied by the scale) that counts once
 // in the softmax's denominator and has no value.
+// As me_attention_decode_bf16 with a window, and beside the window's keys the pooled entries of the blocks of pool_block positions
+// that the window has wholly left behind (pages k_pool, v_pool laid out as the keys' and values': entry b at page table[b / bs],
+// slot b % bs). The result's rows are out_row elements apart (0: nh * d), begin at column out_col and are multiplied by out_scale.
+extern "C" int me_attention_decode_bf16_pooled(const void* q, const void* k_cache, const void* v_cache, const void* k_pool,
+                                               const void* v_pool, int pool_block, const int* item_ctx, const int* block_table,
+                                               int table_width, void* out, long long out_row, int out_col, float out_scale,
+                                               float* part_o, float* part_ml, int items, int nh, int nkv, int d, int bs, int window,
+                                               float scale, int split_keys, int num_splits, int max_ctx, const int* live_items,
+                                               int full_splits, int waves_wanted, const int* step_flags, hipStream_t stream) {
+  DecodeFusedArgs pool{};
+  pool.k_pool = (const bf16_t*)k_pool;
+  pool.v_pool = (const bf16_t*)v_pool;
+  pool.pool_block = pool_block;
+  pool.out_row = out_row;
+  pool.out_col = out_col;
+  pool.out_scale = out_scale;
+  return decode_common(q, k_cache, v_cache, item_ctx, block_table, table_width, out, part_o, part_ml, items, nh, nkv, d, bs, window,
+                       scale, split_keys, num_splits, max_ctx, nullptr, live_items, full_splits, waves_wanted, step_flags, stream, 0,
+                       nullptr, &pool);
+}
+
 extern "C" int me_attention_decode_bf16_sink(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
                                              const int* block_table, int table_width, void* out, float* part_o,
                                              float* part_ml, int items, int nh, int nkv, int d, int bs, const float* sink,
@@ -731,8 +783,15 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
                          const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
                          int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
                          int max_ctx, const DecodeFusedArgs* fused, const int* live_items, int full_splits,
-                         int waves_wanted, const int* step_flags, hipStream_t stream, int keep_first, const float* sink) {
+                         int waves_wanted, const int* step_flags, hipStream_t stream, int keep_first, const float* sink,
+                         const DecodeFusedArgs* pool) {
   if (items <= 0) return 0;
+  if (pool && (fused || keep_first > 0 || sink || window <= 0 || pool->pool_block < 0 || (pool->pool_block > 0 && (!pool->k_pool || !pool->v_pool))))
+    return me_fail("me_attention_decode_bf16: pooled blocks of %d keys need a window, pages of their own, the unfused form, no kept "
+                   "first keys and no sink", pool->pool_block);
+  if (pool && (pool->out_col < 0 || (pool->out_row > 0 && pool->out_col + (long long)nh * d > pool->out_row) || (pool->out_row > 0 && !out)))
+    return me_fail("me_attention_decode_bf16: the result at column %d of a row of %lld", pool->out_col, pool->out_row);
+  if (pool && ((pool->out_row | pool->out_col) & 3)) return me_fail("me_attention_decode_bf16: the result's rows and column are multiples of 4");
   if (keep_first < 0 || (keep_first > 0 && (window <= 0 || fused)))
     return me_fail("me_attention_decode_bf16: keep_first=%d needs a window and the unfused form", keep_first);
   if (!me_attention_mfma_supported(d, bs))
@@ -773,7 +832,7 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   case DD:                                                                                                      \
     launch_decode<DD>(qq, kc, vc, item_ctx, block_table, table_width, part_o, part_ml, items, nh, nkv, bs, window, sl, \
                       depth, num_splits, block_waves, (bf16_t*)out, fused, live_items, waves_wanted, streamed, step_flags, \
-                      keep_first, sink, stream);                                                                \
+                      keep_first, sink, pool, stream);                                                          \
     break;
   switch (d) {
     ME_DECODE_CASE(32)
@@ -787,7 +846,9 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   if (me_check_launch("me_attention_decode_bf16")) return 1;
   if (block_waves > 1) return 0;  // the blocks held all splits of their heads and wrote the output themselves
   if (!out) return 0;             // the caller adds up the splits (me_attention_out_product_bf16)
-  attention_decode_combine_kernel<<<items * nh, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, num_splits, d, sink, nh);
+  attention_decode_combine_kernel<<<items * nh, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, num_splits, d, sink, nh,
+                                                                  pool ? pool->out_row : 0, pool ? pool->out_col : 0,
+                                                                  pool ? pool->out_scale : 1.f);
   return me_check_launch("me_attention_decode_combine");
 }
 
@@ -1041,6 +1102,20 @@ __device__ __forceinline__ void pf_softmax_pv64(const bf16_t* __restrict__ vs, i
 // attention_prefill_combine_kernel adds up; `chunk` is -1 for a tile in one piece. A block runs the
 // entries from its first one (bundle_first[block]) up to and including the next one marked `last`: the
 // host packs entries into bundles of about equal work when a step has too few tiles to go round.
+// Pooled entries beside a window (k_pool null: none): entry b is the mean of the keys (and of the values) at the positions
+// b block .. b block + block - 1, at page table[b / bs], slot b % bs of pages laid out as the keys' and values'. A query at
+// position p sees the entries below (p - window + 1) / block. An entry of the work list whose `last` has bit 1 set walks pooled
+// entries (key_begin, key_last count them) instead of keys. The finished output's rows are out_row elements apart (0: nh * D),
+// begin at column out_col and are multiplied by out_scale.
+struct PrefillPool {
+  const bf16_t* k_pool;
+  const bf16_t* v_pool;
+  int block;
+  long long out_row;
+  int out_col;
+  float out_scale;
+};
+
 struct PrefillWork {
   int item;
   int token_begin, token_count;  // the tile's tokens among the packed tokens of the step
@@ -1048,7 +1123,7 @@ struct PrefillWork {
   int key_begin;                 // first key, a multiple of 64
   int key_last;                  // last key, inclusive
   int chunk;
-  int last;
+  int last;  // bit 0: the bundle ends with this entry; bit 1: the keys are pooled entries
 };
 
 // WAVES waves per block, NB blocks of 16 query columns per wave: WAVES * NB * 16 = 128 columns.
@@ -1058,7 +1133,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     const PrefillWork* __restrict__ work, const int* __restrict__ bundle_first, const int* __restrict__ block_table,
     int table_width, bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks,
     int nh, int nkv, int bs_shift, int window, float scale_log2, int tokens_per_block, int keep_first,
-    const float* __restrict__ sink) {
+    const float* __restrict__ sink, PrefillPool pool) {
   constexpr int THREADS = WAVES * 64;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw);
@@ -1075,6 +1150,10 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
   const int item = w.item;
   const int t_begin = w.token_begin, t_end = w.token_begin + w.token_count;
   const int* table = block_table + (size_t)item * table_width;
+  const bool of_pool = (w.last & 2) != 0;  // the same for every lane
+  const bf16_t* __restrict__ kc = of_pool ? pool.k_pool : k_cache;
+  const bf16_t* __restrict__ vc = of_pool ? pool.v_pool : v_cache;
+  const int win = of_pool ? 0 : window, keep = of_pool ? 0 : keep_first;
 
   // this lane's query column in each of the wave's blocks
   int tok[NB], head[NB], qpos[NB], lo_col[NB];
@@ -1087,7 +1166,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     head[nb] = kvh * group + c % group;
     col_ok[nb] = c < tokens_per_block * group && tok[nb] < t_end;
     qpos[nb] = col_ok[nb] ? w.pos_first + c / group : -1;
-    lo_col[nb] = window > 0 ? max(qpos[nb] - window + 1, 0) : 0;
+    if (of_pool) qpos[nb] = qpos[nb] - window + 1 >= pool.block ? (qpos[nb] - window + 1) / pool.block - 1 : -1;  // the last entry seen
+    lo_col[nb] = win > 0 ? max(qpos[nb] - win + 1, 0) : 0;
     wave_max_pos = max(wave_max_pos, qpos[nb]);
     if (col_ok[nb]) wave_min_pos = min(wave_min_pos, qpos[nb]);
   }
@@ -1122,7 +1202,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
   const int first_tile = w.key_begin;
   const int last_key = w.key_last;
   pf_fetch_pages<D, WAVES>(stage, first_tile, wave, table, table_width, bs_shift);
-  pf_issue_tile<D, WAVES>(stage, first_tile, wave, lds, bs_shift, nkv, kvh, k_cache, v_cache);
+  pf_issue_tile<D, WAVES>(stage, first_tile, wave, lds, bs_shift, nkv, kvh, kc, vc);
   pf_fetch_pages<D, WAVES>(stage, first_tile + PF_KT, wave, table, table_width, bs_shift);
   __syncthreads();
   int buf = 0;
@@ -1132,16 +1212,16 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     const bool active = key0 <= wave_max_pos;  // else every column of the wave lies before this tile
     // Tiles are fetched unconditionally (the page index is clamped to the table, so a tile past the last
     // key reads valid memory that nobody uses).
-    pf_issue_tile<D, WAVES>(stage, key0 + PF_KT, wave, lds + (size_t)(buf ^ 1) * L::BUF_ELEMS, bs_shift, nkv, kvh, k_cache, v_cache);
+    pf_issue_tile<D, WAVES>(stage, key0 + PF_KT, wave, lds + (size_t)(buf ^ 1) * L::BUF_ELEMS, bs_shift, nkv, kvh, kc, vc);
     pf_fetch_pages<D, WAVES>(stage, key0 + 2 * PF_KT, wave, table, table_width, bs_shift);  // for the next iteration
     float4_t s[NB][4];
     pf_scores64<D, NB>(ks, r, g, qf, s);  // also by a wave that will not use them: no control flow around s
     if (active) {
-      const bool need_mask = key0 + PF_KT - 1 > wave_min_pos || window > 0;
+      const bool need_mask = key0 + PF_KT - 1 > wave_min_pos || win > 0;
       if (need_mask)
-        pf_softmax_pv64<D, NB, true>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc, keep_first);
+        pf_softmax_pv64<D, NB, true>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc, keep);
       else
-        pf_softmax_pv64<D, NB, false>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc, keep_first);
+        pf_softmax_pv64<D, NB, false>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc, keep);
     }
     __syncthreads();
   }
@@ -1164,13 +1244,14 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
       if (!col_ok[nb]) continue;
-      float inv = 1.f / lsum[nb];
+      float inv = pool.out_scale / lsum[nb];
       if (sink) {  // one more term exp(sink) in the denominator, with no value (statistics are in units of log2)
         const float s2 = sink[head[nb]] * LOG2E, top = fmaxf(m[nb], s2);
         const float keep = fast_exp2(m[nb] - top);
-        inv = keep / (lsum[nb] * keep + fast_exp2(s2 - top));
+        inv = pool.out_scale * keep / (lsum[nb] * keep + fast_exp2(s2 - top));
       }
-      bf16_t* orow = out + ((size_t)tok[nb] * nh + head[nb]) * D;
+      bf16_t* orow = pool.out_row > 0 ? out + (size_t)tok[nb] * pool.out_row + pool.out_col + (size_t)head[nb] * D
+                                      : out + ((size_t)tok[nb] * nh + head[nb]) * D;
 #pragma unroll
       for (int dt = 0; dt < D / 16; ++dt) {
         const short4_t o = pack_bf16x4(acc[nb][dt][0] * inv, acc[nb][dt][1] * inv, acc[nb][dt][2] * inv,
@@ -1179,7 +1260,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
       }
     }
   }
-  if (w.last) break;  // (the loop over keys ended with a barrier: LDS is free for the next entry)
+  if (w.last & 1) break;  // (the loop over keys ended with a barrier: LDS is free for the next entry)
   }
 }
 
@@ -1191,7 +1272,8 @@ __global__ __launch_bounds__(256) void attention_prefill_combine_kernel(const fl
                                                                         const float* __restrict__ part_ml,
                                                                         const int* __restrict__ token_chunks,
                                                                         bf16_t* __restrict__ out, int nh, int d,
-                                                                        int max_chunks, const float* __restrict__ sink) {
+                                                                        int max_chunks, const float* __restrict__ sink,
+                                                                        long long out_row, int out_col, float out_scale) {
   const int tok = blockIdx.x;
   const int nc = token_chunks[tok];
   if (nc <= 1) return;
@@ -1220,8 +1302,9 @@ __global__ __launch_bounds__(256) void attention_prefill_combine_kernel(const fl
         total[3] = fmaf(wgt, o[3], total[3]);
       }
     }
-    const float inv = 1.f / denom;
-    *reinterpret_cast<short4_t*>(out + unit * d + e) =
+    const float inv = denom > 0.f ? out_scale / denom : 0.f;
+    bf16_t* orow = out_row > 0 ? out + (size_t)tok * out_row + out_col + (size_t)head * d : out + unit * d;
+    *reinterpret_cast<short4_t*>(orow + e) =
         pack_bf16x4(total[0] * inv, total[1] * inv, total[2] * inv, total[3] * inv);
   }
 }
@@ -1239,7 +1322,7 @@ template <int D, int NB>
 static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const PrefillWork* work,
                           const int* bundle_first, const int* table, int width, bf16_t* out,
                           float* part_o, float* part_ml, int max_chunks, int nh, int nkv, int bs_shift, int window,
-                          float sl, int tpb, int keep_first, const float* sink, hipStream_t stream) {
+                          float sl, int tpb, int keep_first, const float* sink, const PrefillPool& pool, hipStream_t stream) {
   static bool configured = false;  // raise the dynamic LDS limit of this instantiation once
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<D, NB, PF_WAVES>),
@@ -1250,7 +1333,7 @@ static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf
   }
   attention_prefill_kernel<D, NB, PF_WAVES><<<grid, PF_WAVES * 64, PrefillLds<D>::BYTES, stream>>>(
       q, kc, vc, work, bundle_first, table, width, out, part_o, part_ml, max_chunks, nh, nkv, bs_shift, window, sl, tpb,
-      keep_first, sink);
+      keep_first, sink, pool);
   return 0;
 }
 
@@ -1271,8 +1354,15 @@ static int prefill_common(const void* q, const void* k_cache, const void* v_cach
                           const int* bundle_first, int num_bundles, float* part_o, float* part_ml,
                           const int* token_chunks, int max_chunks, int num_tokens, int nh, int nkv,
                           int d, int bs, int window, int keep_first, float scale, int columns, const float* sink,
-                          hipStream_t stream) {
+                          hipStream_t stream, const PrefillPool* pooled = nullptr) {
   const int num_work = num_bundles;
+  PrefillPool pool{nullptr, nullptr, 0, 0, 0, 1.f};
+  if (pooled) pool = *pooled;
+  if (pool.block < 0 || (pool.block > 0 && (window <= 0 || keep_first > 0 || sink || !pool.k_pool || !pool.v_pool)))
+    return me_fail("me_attention_prefill_bf16: pooled blocks of %d keys need a window, pages of their own, no kept first keys and no "
+                   "sink", pool.block);
+  if (pool.out_col < 0 || (pool.out_row > 0 && pool.out_col + (long long)nh * d > pool.out_row) || ((pool.out_row | pool.out_col) & 3))
+    return me_fail("me_attention_prefill_bf16: the result at column %d of a row of %lld (multiples of 4)", pool.out_col, pool.out_row);
   if (keep_first < 0 || (keep_first > 0 && window <= 0))
     return me_fail("me_attention_prefill_bf16: keep_first=%d needs a window", keep_first);
   if (num_items <= 0 || num_work <= 0) return 0;
@@ -1302,10 +1392,10 @@ static int prefill_common(const void* q, const void* k_cache, const void* v_cach
   case DD:                                                                                                         \
     rc = wide ? launch_prefill<DD, 2>(grid, qq, kc, vc, (const PrefillWork*)work, bundle_first, block_table,       \
                                       table_width, (bf16_t*)out, part_o, part_ml, max_chunks, nh, nkv, bs_shift,   \
-                                      window, sl, tpb, keep_first, sink, stream)                                   \
+                                      window, sl, tpb, keep_first, sink, pool, stream)                             \
               : launch_prefill<DD, 1>(grid, qq, kc, vc, (const PrefillWork*)work, bundle_first, block_table,       \
                                       table_width, (bf16_t*)out, part_o, part_ml, max_chunks, nh, nkv, bs_shift,   \
-                                      window, sl, tpb, keep_first, sink, stream);                                  \
+                                      window, sl, tpb, keep_first, sink, pool, stream);                            \
     break;
   switch (d) {
     ME_PREFILL_CASE(32)
@@ -1320,7 +1410,7 @@ static int prefill_common(const void* q, const void* k_cache, const void* v_cach
   if (me_check_launch("me_attention_prefill_bf16")) return 1;
   if (max_chunks > 1) {
     attention_prefill_combine_kernel<<<num_tokens, 256, 0, stream>>>(part_o, part_ml, token_chunks, (bf16_t*)out, nh, d,
-                                                                     max_chunks, sink);
+                                                                     max_chunks, sink, pool.out_row, pool.out_col, pool.out_scale);
     return me_check_launch("me_attention_prefill_combine");
   }
   return 0;
@@ -1335,6 +1425,20 @@ extern "C" int me_attention_prefill_bf16_kept(const void* q, const void* k_cache
   return prefill_common(q, k_cache, v_cache, num_items, block_table, table_width, out, work, bundle_first, num_bundles, part_o,
                         part_ml, token_chunks, max_chunks, num_tokens, nh, nkv, d, bs, window, keep_first, scale, columns, nullptr,
                         stream);
+}
+
+// With a window, and beside the window's keys the pooled entries of the blocks of pool_block positions that a query's window
+// has wholly left behind (see PrefillPool); the work list has entries of their own for them (me_prefill_work_list_pooled).
+extern "C" int me_attention_prefill_bf16_pooled(const void* q, const void* k_cache, const void* v_cache, const void* k_pool,
+                                                const void* v_pool, int pool_block, int num_items, const int* block_table,
+                                                int table_width, void* out, long long out_row, int out_col, float out_scale,
+                                                const int* work, const int* bundle_first, int num_bundles, float* part_o,
+                                                float* part_ml, const int* token_chunks, int max_chunks, int num_tokens, int nh,
+                                                int nkv, int d, int bs, int window, float scale, int columns, hipStream_t stream) {
+  const PrefillPool pool{(const bf16_t*)k_pool, (const bf16_t*)v_pool, pool_block, out_row, out_col, out_scale};
+  return prefill_common(q, k_cache, v_cache, num_items, block_table, table_width, out, work, bundle_first, num_bundles, part_o,
+                        part_ml, token_chunks, max_chunks, num_tokens, nh, nkv, d, bs, window, 0, scale, columns, nullptr, stream,
+                        &pool);
 }
 
 // All keys visible, with a sink (see prefill_common).

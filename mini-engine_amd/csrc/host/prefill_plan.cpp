@@ -21,6 +21,8 @@ struct Tile {
   int item, first_token, tokens, first_pos, first_key, last_pos, key_tiles;
   int kept_tiles = 0;  // key tiles of the kept first keys that the tile's window has left behind: they come before the window's
                        // in the tile's order of key tiles, and lie at keys 0 .. 64 * kept_tiles - 1
+  int pooled = 0;      // with pooled blocks: the pooled entries that the tile's last token sees (those of the blocks its window
+                       // has wholly left behind); their key tiles take the kept keys' place, and walk entries instead of keys
 };
 struct Piece {
   int length, tile, chunk, first_tile;  // chunk -1: the tile in one piece
@@ -37,7 +39,9 @@ std::vector<Piece> cut(const std::vector<Tile>& tiles, int cap) {
       continue;
     }
     int j = 0;  // (no piece reaches across the gap between the kept keys and the window)
-    for (int t0 = 0; t0 < kept; t0 += cap, ++j) pieces.push_back({std::min(cap, kept - t0), i, j, t0});
+    // (pooled entries stay in one piece: a tile then has at most one chunk more than its window's keys give it)
+    const int kept_cap = tiles[i].pooled > 0 ? kept : cap;
+    for (int t0 = 0; t0 < kept; t0 += kept_cap, ++j) pieces.push_back({std::min(kept_cap, kept - t0), i, j, t0});
     for (int t0 = 0; t0 < n; t0 += cap, ++j) pieces.push_back({std::min(cap, n - t0), i, j, kept + t0});
   }
   return pieces;
@@ -100,7 +104,7 @@ bool wide_blocks_pay(const int* starts, const int* qlens, int items, int tpb, in
 // results a second kernel adds up, and the pieces are packed into one bundle per compute unit; `cap` is
 // the candidate with the shortest longest bundle, where cutting at all counts as kCutOverhead key tiles.
 void build_work_list(const int* starts, const int* qlens, int items, int tpb, int window, int nkv, int slots,
-                     long long partial_row_bytes, WorkList& out, int keep_first) {
+                     long long partial_row_bytes, WorkList& out, int keep_first, int pool_block) {
   std::vector<Tile> tiles;
   int offset = 0;
   for (int i = 0; i < items; ++i) {
@@ -110,6 +114,10 @@ void build_work_list(const int* starts, const int* qlens, int items, int tpb, in
       const int k0 = window > 0 ? (std::max(p_first - window + 1, 0) / 64) * 64 : 0;
       tiles.push_back({i, offset + t0, count, p_first, k0, p_last, (p_last - k0) / 64 + 1});
       if (window > 0 && keep_first > 0 && k0 > 0) tiles.back().kept_tiles = (std::min(keep_first, k0) + 63) / 64;
+      if (window > 0 && pool_block > 0 && p_last - window + 1 >= pool_block) {
+        tiles.back().pooled = (p_last - window + 1) / pool_block;
+        tiles.back().kept_tiles = (tiles.back().pooled + 63) / 64;
+      }
     }
     offset += qlens[i];
   }
@@ -129,6 +137,7 @@ void build_work_list(const int* starts, const int* qlens, int items, int tpb, in
     long long chunk_limit = 1ll << 30;
     if (partial_row_bytes > 0) chunk_limit = std::max(1ll, kPartialBytesMax / (partial_row_bytes * std::max(1, offset)));
     if (keep_first > 0) chunk_limit = std::max(1ll, chunk_limit - 1);  // (the kept keys' piece is one more)
+    if (pool_block > 0) chunk_limit = std::max(1ll, chunk_limit - 1);  // (and so is the pooled entries' piece)
     std::vector<int> caps = {longest, (int)((total + bins - 1) / bins), (int)((total + 2ll * bins - 1) / (2ll * bins)),
                              (longest + 1) / 2, (longest + 2) / 3};
     std::sort(caps.begin(), caps.end());
@@ -171,11 +180,12 @@ void build_work_list(const int* starts, const int* qlens, int items, int tpb, in
       const Tile& t = tiles[p.tile];
       const bool of_kept = p.first_tile < t.kept_tiles;
       const int begin = of_kept ? 64 * p.first_tile : t.first_key + 64 * (p.first_tile - t.kept_tiles);
-      const int row[8] = {t.item, t.first_token, t.tokens, t.first_pos, begin,
-                          std::min(of_kept ? std::min(keep_first, t.first_key) - 1 : t.last_pos, begin + 64 * p.length - 1), p.chunk, 0};
+      const int limit = !of_kept ? t.last_pos + 1 : t.pooled > 0 ? t.pooled : std::min(keep_first, t.first_key);
+      const int row[8] = {t.item, t.first_token, t.tokens, t.first_pos, begin, std::min(limit - 1, begin + 64 * p.length - 1), p.chunk,
+                          of_kept && t.pooled > 0 ? 2 : 0};
       out.work.insert(out.work.end(), row, row + 8);
     }
-    out.work.back() = 1;  // the bundle ends with this entry
+    out.work.back() |= 1;  // the bundle ends with this entry
   }
   out.max_chunks = 1;
   for (size_t i = 0; i < tiles.size(); ++i) {
@@ -194,6 +204,23 @@ extern "C" {
 // bundle, token_chunks one per token; counts: entries, bundles, max chunks. Returns 0, or -1 when a buffer is
 // too small (counts then say what is needed).
 // keep_first: with a window, the first keys that stay visible behind it (an entry of their own per tile that has left them).
+// pool_block: with a window, the pooled entries of the blocks of that many positions that a tile's window has wholly left behind
+// (entries of their own, marked by bit 1 of their last field, whose keys count pooled entries).
+int me_prefill_work_list_pooled(const int32_t* starts, const int32_t* qlens, int items, int tpb, int window, int pool_block, int nkv,
+                                int slots, long long partial_row_bytes, int32_t* work, int cap_entries, int32_t* bundle_first,
+                                int cap_bundles, int32_t* token_chunks, int cap_tokens, int32_t* counts) {
+  me::WorkList list;
+  me::build_work_list(starts, qlens, items, tpb, window, nkv, slots, partial_row_bytes, list, 0, pool_block);
+  counts[0] = (int)list.work.size() / 8;
+  counts[1] = (int)list.bundle_first.size();
+  counts[2] = list.max_chunks;
+  if (counts[0] > cap_entries || counts[1] > cap_bundles || (int)list.token_chunks.size() > cap_tokens) return -1;
+  std::copy(list.work.begin(), list.work.end(), work);
+  std::copy(list.bundle_first.begin(), list.bundle_first.end(), bundle_first);
+  std::copy(list.token_chunks.begin(), list.token_chunks.end(), token_chunks);
+  return 0;
+}
+
 int me_prefill_work_list_kept(const int32_t* starts, const int32_t* qlens, int items, int tpb, int window, int keep_first, int nkv,
                               int slots, long long partial_row_bytes, int32_t* work, int cap_entries, int32_t* bundle_first,
                               int cap_bundles, int32_t* token_chunks, int cap_tokens, int32_t* counts) {

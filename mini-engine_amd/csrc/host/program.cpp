@@ -167,6 +167,14 @@ bool attention_takes_tiled_prefill(const Op& op, int dtype) {
   return dtype == kBF16 && (op.i[9] == 0 || op.i[9] == d) && me_attention_mfma_supported(d, bs) && nh / nkv <= 16;
 }
 
+// Whether an attention operation over a window and pooled blocks goes to the matrix-core kernels: bfloat16, keys and values of
+// one size that the kernels are built for, up to 16 heads to a key/value head, results at rows and a column that are multiples of 4.
+bool pooled_takes_matrix_cores(const Op& op, int dtype, long long out_row) {
+  const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2], dv = (int)op.i[3], bs = (int)op.i[4];
+  return dtype == kBF16 && dv == d && op.i[5] > 0 && me_attention_mfma_supported(d, bs) && nh / nkv <= 16 && out_row % 4 == 0 &&
+         op.i[11] % 4 == 0;
+}
+
 int groups_of(int64_t v) { return v > 1 ? (int)v : 1; }
 float scale_of(float f) { return f == 0.f ? 1.f : f; }
 
@@ -809,9 +817,39 @@ class Run {
     ok(me_whole_norm_scatter(bufs_[op.in], row, (int)op.i[8], (int)op.i[9], (int)op.i[10], (const float*)op.p[0], (const float*)op.p[1],
                              idx(s_.lay.positions), idx(s_.lay.token_item), table, width, q, (void*)op.p[2], (void*)op.p[3],
                              (void*)op.p[4], (void*)op.p[5], t_, nh, nkv, d, dv, bs, pool, op.f[0], dtype_, stream_));
+    const float out_scale = op.f[2];  // (always given; nought is a scale like any other)
+    if (pooled_takes_matrix_cores(op, dtype_, out_row) && s_.decode_only) {
+      // one new token per item: the split-context kernel, which deals the pooled entries' tiles to its splits before the window's
+      const int items = s_.lay.items;
+      if ((long long)width * bs < s_.max_ctx) throw Error(kBadValue, "the block table cannot hold the step's longest context");
+      const SplitPlan sp = split_plan(items, nkv * ((nh / nkv + 15) / 16), s_.max_ctx, s_.least_live, idx(s_.lay.live_items));
+      float* part_o = (float*)arena_.take((size_t)items * nh * sp.num_splits * d * 4);
+      float* part_ml = (float*)arena_.take((size_t)items * nh * sp.num_splits * 2 * 4);
+      ok(me_attention_decode_bf16_pooled(q, op.p[2], op.p[3], op.p[4], op.p[5], pool, idx(s_.lay.item_ctx), table, width, bufs_[op.out],
+                                         out_row, (int)op.i[11], out_scale, part_o, part_ml, items, nh, nkv, d, bs, window, op.f[1],
+                                         sp.split_keys, sp.num_splits, s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves,
+                                         idx(s_.lay.live_items) + 1, stream_));
+      return;
+    }
+    if (pooled_takes_matrix_cores(op, dtype_, out_row)) {
+      // prompts and portions: the tiled kernel, whose work list has an entry of its own for a tile's pooled entries
+      auto it = s_.plans.find({nh, nkv, d, window, 0, pool});
+      if (it == s_.plans.end()) throw Error(kBroken, "the step has no work list for an attention layer with pooled blocks");
+      const StepView::Plan& p = it->second;
+      float *part_o = nullptr, *part_ml = nullptr;
+      if (p.max_chunks > 1) {
+        part_o = (float*)arena_.take((size_t)t_ * nh * p.max_chunks * d * 4);
+        part_ml = (float*)arena_.take((size_t)t_ * nh * p.max_chunks * 2 * 4);
+      }
+      ok(me_attention_prefill_bf16_pooled(q, op.p[2], op.p[3], op.p[4], op.p[5], pool, s_.lay.items, table, width, bufs_[op.out], out_row,
+                                          (int)op.i[11], out_scale, idx(p.work), idx(p.bundle_first), p.bundles, part_o, part_ml,
+                                          p.token_chunks >= 0 ? idx(p.token_chunks) : nullptr, p.max_chunks, t_, nh, nkv, d, bs, window,
+                                          op.f[1], p.columns, stream_));
+      return;
+    }
     ok(me_attention_general_pooled(q, op.p[2], op.p[3], idx(s_.lay.positions), idx(s_.lay.token_item), table, width, bufs_[op.out], t_, nh,
                                    nkv, d, dv, bs, window, 0, nullptr, 0, op.f[1], nullptr, nullptr, 0, op.p[4], op.p[5], pool, out_row,
-                                   (int)op.i[11], scale_of(op.f[2]), dtype_, s_.lay.items, stream_));
+                                   (int)op.i[11], out_scale, dtype_, s_.lay.items, stream_));
   }
 
   // Linear attention by the generalized delta rule over the state rows of the step's items (csrc/delta_rule.hip).
@@ -819,7 +857,7 @@ class Run {
     ok(me_delta_rule(bufs_[op.in], values_[op.in].cols, (int)op.i[3], (int)op.i[4], (int)op.i[5], (int)op.i[6], (int)op.i[7], (int)op.i[8],
                      op.p[0], (const float*)op.p[1], (const float*)op.p[2], (const float*)op.p[3], (float*)op.p[4],
                      idx(s_.lay.item_start), idx(s_.lay.state_slots), bufs_[op.out], values_[op.out].cols, (int)op.i[9],
-                     scale_of(op.f[2]), t_, s_.lay.items, (int)op.i[0], (int)op.i[1], (int)op.i[2], op.f[0], op.f[1], dtype_, stream_));
+                     op.f[2], t_, s_.lay.items, (int)op.i[0], (int)op.i[1], (int)op.i[2], op.f[0], op.f[1], dtype_, stream_));
   }
 
   // Rows are selected before the final norm, as the reference does (model.py:186); logits are float32.
@@ -927,6 +965,10 @@ std::vector<std::vector<int>> Program::prefill_geometries() const {
       std::vector<int> key = {(int)op.i[0], 1, (int)(op.i[3] + op.i[2]), 0, 0};
       if (std::find(out.begin(), out.end(), key) == out.end()) out.push_back(key);
     }
+    if (op.kind == kOpPooledAttention && pooled_takes_matrix_cores(op, dtype_, values_[op.out].cols)) {
+      std::vector<int> key = {(int)op.i[0], (int)op.i[1], (int)op.i[2], (int)op.i[5], 0, (int)op.i[6]};
+      if (std::find(out.begin(), out.end(), key) == out.end()) out.push_back(key);
+    }
     if (op.kind != kOpAttention) continue;
     const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2], bs = (int)op.i[4], window = (int)op.i[5];
     if (!attention_is_plain(op) && !attention_takes_tiled_prefill(op, dtype_)) continue;
@@ -968,7 +1010,22 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
     if (op.kind == kOpRoutedFF)
       need = (size_t)(op.i[1] + 1) * tokens * hidden_ * 4 + (size_t)me_routed_ff_workspace(tokens, (int)op.i[0], (int)op.i[1], (int)op.i[2], (int)elem) +
              (size_t)tokens * (4 + 3 * op.i[7] * elem + 2 * op.i[7] * 4) + 6 * pad;
-    if (op.kind == kOpPooledAttention) need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;
+    if (op.kind == kOpPooledAttention) {
+      need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;
+      if (dtype_ == kBF16 && op.i[3] == op.i[2] && me_attention_mfma_supported((int)op.i[2], (int)op.i[4]) && op.i[0] / op.i[1] <= 16) {
+        const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2];
+        size_t most = 0;  // the splits' partial results of a decode step
+        for (int64_t b = 1; b <= items; ++b) {
+          int keys, splits;
+          decode_splits((int)std::max<int64_t>(1, (b + 1) / 2), nkv * ((nh / nkv + 15) / 16), (int)max_ctx, keys, splits);
+          most = std::max(most, (size_t)b * splits);
+        }
+        const size_t decode = most * nh * (d + 2) * 4 + 2 * pad;
+        // partial results of cut tiles: the work list's bound, and one chunk more for the pooled entries
+        const size_t prefill = (size_t)(256ll << 20) + (size_t)(256ll << 20) * 2 / d + (size_t)tokens * nh * (d + 2) * 4 * 2 + 2 * pad;
+        need += std::max(decode, tokens > items ? prefill : (size_t)0);
+      }
+    }
     if (op.kind == kOpAttention && !attention_is_plain(op)) {
       need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;
       if (attention_takes_tiled_prefill(op, dtype_)) {  // the splits' partial results of a decode step

@@ -67,6 +67,7 @@ void hip_ok(hipError_t e, const char* what) {
 // The work list of one attention geometry for the current step, from the cache or made now.
 const CachedPlan& plan_for(Runner& r, const std::vector<int>& geometry) {
   const int nh = geometry[0], nkv = geometry[1], d = geometry[2], window = geometry[3], keep_first = geometry[4];
+  const int pool_block = geometry.size() > 5 ? geometry[5] : 0;  // (only geometries with pooled blocks have a sixth number)
   std::vector<int> key = geometry;
   key.insert(key.end(), r.starts.begin(), r.starts.end());
   key.push_back(-1);
@@ -85,7 +86,7 @@ const CachedPlan& plan_for(Runner& r, const std::vector<int>& geometry) {
                                                    std::max(1, me_attention_prefill_columns(1) / group), window, nkv, r.compute_units);
   fresh.columns = me_attention_prefill_columns(wide ? 1 : 0);
   me::build_work_list(r.starts.data(), r.qlens.data(), items, fresh.columns / group, window, nkv, r.compute_units,
-                      (long long)nh * d * 4, fresh.list, keep_first);
+                      (long long)nh * d * 4, fresh.list, keep_first, pool_block);
   r.plans.push_front(std::move(fresh));
   if (r.plans.size() > 64) r.plans.pop_back();
   return r.plans.front();

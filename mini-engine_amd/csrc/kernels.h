@@ -90,6 +90,18 @@ int me_attention_decode_bf16_kept(const void* q, const void* k_cache, const void
                                   int nh, int nkv, int d, int bs, int window, int keep_first, float scale, int split_keys,
                                   int num_splits, int max_ctx, const int* live_items, int full_splits, int waves_wanted,
                                   const int* step_flags, hipStream_t stream);
+int me_attention_prefill_bf16_pooled(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
+                                     int pool_block, int num_items, const int* block_table, int table_width, void* out,
+                                     long long out_row, int out_col, float out_scale, const int* work, const int* bundle_first,
+                                     int num_bundles, float* part_o, float* part_ml, const int* token_chunks, int max_chunks,
+                                     int num_tokens, int nh, int nkv, int d, int bs, int window, float scale, int columns,
+                                     hipStream_t stream);
+int me_attention_decode_bf16_pooled(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
+                                    int pool_block, const int* item_ctx, const int* block_table, int table_width, void* out,
+                                    long long out_row, int out_col, float out_scale, float* part_o, float* part_ml, int items, int nh,
+                                    int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits, int max_ctx,
+                                    const int* live_items, int full_splits, int waves_wanted, const int* step_flags,
+                                    hipStream_t stream);
 int me_attention_general_gated(const void* q, const void* k_cache, const void* v_cache, const int* positions,
                                const int* token_item, const int* block_table, int table_width, void* out, int num_tokens, int nh,
                                int nkv, int d, int dv, int bs, int window, int keep_first, const float* unturn, int un_pairing,

@@ -1057,7 +1057,7 @@ class PrefillPlan:
 
 
 def prefill_work_list(starts: list[int], qlens: list[int], tpb: int, window: int, nkv: int, slots: int,
-                      partial_row_bytes: int = 0, keep_first: int = 0):
+                      partial_row_bytes: int = 0, keep_first: int = 0, pooled_block: int = 0):
     """Host side of :class:`PrefillPlan`: (entries int32 [n, 8], first entry of each bundle int32 [b],
     chunks per token int32 [T], max chunks), as ``csrc/host/prefill_plan.cpp`` builds it (the native
     step uses the same builder).
@@ -1067,7 +1067,11 @@ def prefill_work_list(starts: list[int], qlens: list[int], tpb: int, window: int
     tiles of a step with few of them are cut into key ranges whose partial results a second kernel adds
     up. An entry is (item, first token, tokens, first position, first key, last key, chunk or -1, 1 if
     its bundle ends with it). With ``keep_first`` (and a window) a tile whose window has left the first keys behind
-    has an entry of its own for the keys ``0 .. min(keep_first, its window's first tile) - 1``, so it always has chunks."""
+    has an entry of its own for the keys ``0 .. min(keep_first, its window's first tile) - 1``, so it always has chunks.
+    With ``pooled_block`` P (and a window) a tile whose last token sees pooled entries (those of the blocks of P positions that
+    its window has wholly left behind) has one entry for them; its keys count entries and its last field has bit 1 set."""
+    if keep_first and pooled_block:
+        raise ValueError("kept first keys and pooled blocks do not go together")
     s = np.ascontiguousarray(starts, dtype=np.int32)
     q = np.ascontiguousarray(qlens, dtype=np.int32)
     total = int(q.sum())
@@ -1077,8 +1081,9 @@ def prefill_work_list(starts: list[int], qlens: list[int], tpb: int, window: int
         work = np.empty((cap_entries, 8), dtype=np.int32)
         first = np.empty(cap_bundles, dtype=np.int32)
         token_chunks = np.empty(total, dtype=np.int32)
-        rc = lib().me_prefill_work_list_kept(_vp(s.ctypes.data), _vp(q.ctypes.data), _i(len(q)), _i(tpb), _i(window),
-                                             _i(keep_first), _i(nkv), _i(slots), ctypes.c_longlong(partial_row_bytes),
+        fn = lib().me_prefill_work_list_pooled if pooled_block else lib().me_prefill_work_list_kept
+        rc = fn(_vp(s.ctypes.data), _vp(q.ctypes.data), _i(len(q)), _i(tpb), _i(window),
+                                             _i(pooled_block if pooled_block else keep_first), _i(nkv), _i(slots), ctypes.c_longlong(partial_row_bytes),
                                              _vp(work.ctypes.data), _i(cap_entries), _vp(first.ctypes.data), _i(cap_bundles),
                                              _vp(token_chunks.ctypes.data), _i(total), _vp(counts.ctypes.data))
         if rc == 0:
@@ -1091,14 +1096,14 @@ _PLANS: dict = {}  # the last plans made, by what they were made from: steps of 
 
 
 def prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int, window: int, device,
-                 wide: bool | None = None, keep_first: int = 0) -> PrefillPlan:
+                 wide: bool | None = None, keep_first: int = 0, pooled_block: int = 0) -> PrefillPlan:
     """``wide``: blocks of twice as many query columns or not; None lets the step's size decide."""
-    key = (tuple(starts), tuple(qlens), nh, nkv, d, window, str(device), wide, keep_first)
+    key = (tuple(starts), tuple(qlens), nh, nkv, d, window, str(device), wide, keep_first, pooled_block)
     plan = _PLANS.get(key)
     if plan is None:
         if len(_PLANS) >= 64:
             _PLANS.pop(next(iter(_PLANS)))
-        plan = _PLANS[key] = _make_prefill_plan(starts, qlens, nh, nkv, d, window, device, wide, keep_first)
+        plan = _PLANS[key] = _make_prefill_plan(starts, qlens, nh, nkv, d, window, device, wide, keep_first, pooled_block)
     return plan
 
 
@@ -1123,14 +1128,14 @@ def set_prefill_wide_limits(min_blocks: float, min_key_tiles: float) -> tuple[fl
 
 
 def _make_prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int, window: int, device,
-                       wide: bool | None = None, keep_first: int = 0) -> PrefillPlan:
+                       wide: bool | None = None, keep_first: int = 0, pooled_block: int = 0) -> PrefillPlan:
     group = nh // nkv
     slots = torch.cuda.get_device_properties(device).multi_processor_count
     if wide is None:
         wide = wide_blocks_pay(starts, qlens, max(1, lib().me_attention_prefill_columns(1) // group), window, nkv, slots)
     columns = lib().me_attention_prefill_columns(1 if wide else 0)
     tpb = columns // group
-    work, first, token_chunks, max_chunks = prefill_work_list(starts, qlens, tpb, window, nkv, slots, nh * d * 4, keep_first)
+    work, first, token_chunks, max_chunks = prefill_work_list(starts, qlens, tpb, window, nkv, slots, nh * d * 4, keep_first, pooled_block)
     parts = [work.reshape(-1), first] + ([token_chunks] if max_chunks > 1 else [])
     both = torch.from_numpy(np.concatenate(parts)).to(device)  # one upload
     a, b = work.size, work.size + first.size
@@ -1413,6 +1418,54 @@ def attention_pooled(q, k_cache, v_cache, k_pool, v_pool, positions, token_item,
         _i(nh), _i(nkv), _i(d), _i(dv), _i(bs), _i(window), _i(0), _p(None), _i(0), _f(scale), _p(None), _p(None), _i64(0),
         _p(k_pool), _p(v_pool), _i(pooled_block), _i64(out.shape[1]), _i(out_col), _f(out_scale), _i(_code(q.dtype)),
         _i(block_table.shape[0]), _stream()))
+    return out
+
+
+def attention_pooled_mfma_supported(d: int, dv: int, block_size: int, group: int) -> bool:
+    """Whether :func:`attention_pooled_bf16` takes these sizes (bfloat16 only)."""
+    return d == dv and attention_mfma_supported(d, block_size, group)
+
+
+def attention_pooled_bf16(q, k_cache, v_cache, k_pool, v_pool, positions, item_start, starts: list[int], qlens: list[int], block_table,
+                          scale: float, window: int, pooled_block: int, out: torch.Tensor | None = None, out_col: int = 0,
+                          out_scale: float = 1.0) -> torch.Tensor:
+    """What :func:`attention_pooled` computes, in bfloat16 on the matrix cores: the split-context kernel when every item brings
+    one token (the pooled entries' tiles are dealt to the splits before the window's), else the tiled kernel (a tile's pooled
+    entries are an entry of the work list of their own). ``starts``: the position of each item's first token."""
+    _want(q, "q", torch.bfloat16, (None, None, None))
+    t, nh, d = q.shape
+    nkv, bs = k_cache.shape[1], k_cache.shape[2]
+    _check_cache(k_cache, v_cache, torch.bfloat16, nkv, d, bs)
+    _want(k_pool, "k_pool", torch.bfloat16, tuple(k_cache.shape))
+    _want(v_pool, "v_pool", torch.bfloat16, tuple(v_cache.shape))
+    items = len(qlens)
+    _want(block_table, "block_table", torch.int32, (items, None))
+    if out is None:
+        out = torch.empty((t, nh * d), dtype=torch.bfloat16, device=q.device)
+    _want(out, "out", torch.bfloat16, (t, None))
+    if all(n == 1 for n in qlens):
+        max_ctx = max(starts) + 1
+        item_ctx = torch.tensor([s + 1 for s in starts], dtype=torch.int32, device=q.device)
+        split_keys, num_splits, live_count, full_splits = _decode_split_plan(items, nkv * -(-(nh // nkv) // 16), max_ctx, None)
+        part_o = torch.empty((items * nh * num_splits * d,), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((items * nh * num_splits * 2,), dtype=torch.float32, device=q.device)
+        check(lib().me_attention_decode_bf16_pooled(
+            _p(q), _p(k_cache), _p(v_cache), _p(k_pool), _p(v_pool), _i(pooled_block), _p(item_ctx), _p(block_table),
+            _i(block_table.shape[1]), _p(out), _i64(out.shape[1]), _i(out_col), _f(out_scale), _p(part_o), _p(part_ml), _i(items), _i(nh),
+            _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(split_keys), _i(num_splits), _i(max_ctx), _p(live_count), _i(full_splits),
+            _i(DECODE_WAVES), _p(None), _stream()))
+        return out
+    _want(item_start, "item_start", torch.int32, (items + 1,))
+    plan = prefill_plan(starts, qlens, nh, nkv, d, window, q.device, pooled_block=pooled_block)
+    part_o = part_ml = None
+    if plan.max_chunks > 1:
+        part_o = torch.empty((t * nh * plan.max_chunks * d,), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((t * nh * plan.max_chunks * 2,), dtype=torch.float32, device=q.device)
+    check(lib().me_attention_prefill_bf16_pooled(
+        _p(q), _p(k_cache), _p(v_cache), _p(k_pool), _p(v_pool), _i(pooled_block), _i(items), _p(block_table), _i(block_table.shape[1]),
+        _p(out), _i64(out.shape[1]), _i(out_col), _f(out_scale), _p(plan.work), _p(plan.bundle_first), _i(plan.num_bundles), _p(part_o),
+        _p(part_ml), _p(plan.token_chunks), _i(plan.max_chunks), _i(t), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale),
+        _i(plan.columns), _stream()))
     return out
 
 
