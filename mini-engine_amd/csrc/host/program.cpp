@@ -854,10 +854,21 @@ class Run {
 
   // Linear attention by the generalized delta rule over the state rows of the step's items (csrc/delta_rule.hip).
   void delta_rule(const Op& op) {
+    const int heads = (int)op.i[0], d = (int)op.i[1];
+    if (t_ > s_.lay.items) {
+      // an item brings more than one token: the walk over the tokens does nothing but the recurrence (what every token can
+      // have ahead of it, and what it is owed afterwards, runs for all tokens at once)
+      void* ws = arena_.take((size_t)me_delta_rule_workspace(t_, heads, d));
+      ok(me_delta_rule_steps(bufs_[op.in], values_[op.in].cols, (int)op.i[3], (int)op.i[4], (int)op.i[5], (int)op.i[6], (int)op.i[7],
+                             (int)op.i[8], op.p[0], (const float*)op.p[1], (const float*)op.p[2], (const float*)op.p[3], (float*)op.p[4],
+                             idx(s_.lay.item_start), idx(s_.lay.state_slots), bufs_[op.out], values_[op.out].cols, (int)op.i[9], op.f[2],
+                             t_, s_.lay.items, heads, d, (int)op.i[2], op.f[0], op.f[1], dtype_, ws, stream_));
+      return;
+    }
     ok(me_delta_rule(bufs_[op.in], values_[op.in].cols, (int)op.i[3], (int)op.i[4], (int)op.i[5], (int)op.i[6], (int)op.i[7], (int)op.i[8],
                      op.p[0], (const float*)op.p[1], (const float*)op.p[2], (const float*)op.p[3], (float*)op.p[4],
                      idx(s_.lay.item_start), idx(s_.lay.state_slots), bufs_[op.out], values_[op.out].cols, (int)op.i[9],
-                     op.f[2], t_, s_.lay.items, (int)op.i[0], (int)op.i[1], (int)op.i[2], op.f[0], op.f[1], dtype_, stream_));
+                     op.f[2], t_, s_.lay.items, heads, d, (int)op.i[2], op.f[0], op.f[1], dtype_, stream_));
   }
 
   // Rows are selected before the final norm, as the reference does (model.py:186); logits are float32.
@@ -1010,6 +1021,7 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
     if (op.kind == kOpRoutedFF)
       need = (size_t)(op.i[1] + 1) * tokens * hidden_ * 4 + (size_t)me_routed_ff_workspace(tokens, (int)op.i[0], (int)op.i[1], (int)op.i[2], (int)elem) +
              (size_t)tokens * (4 + 3 * op.i[7] * elem + 2 * op.i[7] * 4) + 6 * pad;
+    if (op.kind == kOpDeltaRule && tokens > items) need = (size_t)me_delta_rule_workspace(tokens, (int)op.i[0], (int)op.i[1]) + pad;
     if (op.kind == kOpPooledAttention) {
       need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;
       if (dtype_ == kBF16 && op.i[3] == op.i[2] && me_attention_mfma_supported((int)op.i[2], (int)op.i[4]) && op.i[0] / op.i[1] <= 16) {

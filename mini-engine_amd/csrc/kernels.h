@@ -187,6 +187,11 @@ int me_delta_rule(const void* proj, long long row, int c_r, int c_k, int c_v, in
                   const float* w0, const float* a_bias, const float* norm_w, float* state, const int* item_start,
                   const int* state_slots, void* out, long long out_row, int out_col, float out_scale, int num_tokens, int items,
                   int heads, int d, int lora, float eps, float decay_coef, int dtype, hipStream_t stream);
+long long me_delta_rule_workspace(long long tokens, int heads, int d);
+int me_delta_rule_steps(const void* proj, long long row, int c_r, int c_k, int c_v, int c_g, int c_a, int c_w1, const void* W2,
+                  const float* w0, const float* a_bias, const float* norm_w, float* state, const int* item_start,
+                  const int* state_slots, void* out, long long out_row, int out_col, float out_scale, int num_tokens, int items,
+                  int heads, int d, int lora, float eps, float decay_coef, int dtype, void* workspace, hipStream_t stream);
 int me_sample_chunks(int vocab);
 int me_sample(const float* logits, int num_rows, int vocab, const float* temperatures, const uint64_t* keys, int* out,
               void* workspace, hipStream_t stream);

@@ -1492,6 +1492,14 @@ def delta_rule(proj: torch.Tensor, cols: dict, w2: torch.Tensor, w0: torch.Tenso
     if out is None:
         out = torch.empty((t, n), dtype=proj.dtype, device=proj.device)
     _want(out, "out", proj.dtype, (t, None))
+    if t > items:  # an item brings more than one token: prepare, scan and finish as kernels of their own
+        lib().me_delta_rule_workspace.restype = ctypes.c_longlong
+        ws = torch.empty(int(lib().me_delta_rule_workspace(_i64(t), _i(heads), _i(d))), dtype=torch.uint8, device=proj.device)
+        check(lib().me_delta_rule_steps(_p(proj), _i64(row), _i(cols["r"]), _i(cols["k"]), _i(cols["v"]), _i(cols["g"]), _i(cols["a"]),
+                                        _i(cols["w1"]), _p(w2), _p(w0), _p(a_bias), _p(norm_w), _p(state), _p(item_start), _p(state_slots),
+                                        _p(out), _i64(out.shape[1]), _i(out_col), _f(out_scale), _i(t), _i(items), _i(heads), _i(d), _i(rank),
+                                        _f(eps), _f(decay_coef), _i(_code(proj.dtype)), _p(ws), _stream()))
+        return out
     check(lib().me_delta_rule(_p(proj), _i64(row), _i(cols["r"]), _i(cols["k"]), _i(cols["v"]), _i(cols["g"]), _i(cols["a"]), _i(cols["w1"]),
                               _p(w2), _p(w0), _p(a_bias), _p(norm_w), _p(state), _p(item_start), _p(state_slots), _p(out),
                               _i64(out.shape[1]), _i(out_col), _f(out_scale), _i(t), _i(items), _i(heads), _i(d), _i(rank), _f(eps),
