@@ -107,20 +107,29 @@ __global__ __launch_bounds__(RPT * DR_PARTS * 4) void delta_rule_kernel(
   }
 }
 
-// ---- steps that bring an item more than one token: three kernels, so that the walk over the tokens, which no token can start
+// ---- steps that bring an item more than one token: four kernels, so that the walk over the tokens, which no token can start
 // before the one ahead of it is done, does nothing but the recurrence.
 //
 //   prepare   every token at once: the decay w_t and the removal rate a_t (the inner product with W_2, sigmoids, the
-//             exponential), and r_t, k_t, v_t as float32, laid out as the walk's lanes read them: the rows part, part + 4, ..
-//             of a lane side by side, so that a lane fetches its rows of a vector sixteen bytes at a time.
-//   scan      a wave of its own for every 16 value channels of an (item, head): the columns of the state do not meet, so the
-//             waves of a head do not wait for each other; the next token's vectors are asked for while this token's are
-//             multiplied (heads of up to 64 rows: both sets fit the registers). The arithmetic is the one of the kernel above,
-//             in its order: a token's state and output have the same bits whichever of the two ran.
+//             exponential), and r_t, k_t, v_t as float32, laid out as the walk's lanes read them.
+//   unit      every (token, head) at once: the unit key u_t and a_t * u_t.
+//   scan      a wave of its own for every 4 value channels of an (item, head): the columns of the state do not meet, so the
+//             waves of a head do not wait for each other, and a head of 64 channels keeps 16 compute units busy. A column
+//             belongs to a row of 16 lanes that hold its rows part, part + 16, ..: sums over the rows are a lane's own sum,
+//             then four exchanges inside the row of lanes (data-parallel moves, no trip through LDS), which leave every lane
+//             of the row with the same bits. The vectors of the tokens ahead are asked for while this token's are multiplied
+//             (SCAN_AHEAD tokens; what a lane holds of a token is a few registers).
 //   finish    every token at once: a head's outputs over their root mean square, the weight, the gate, the scale.
 //
-// Workspace, float32: [T, heads, 5, DP] with DP = 4 RPT >= d (k, r, w, a in the lanes' order, v in its own; rows from d on are
-// nought and leave the state's padding nought), then the raw outputs [T, heads * d].
+// The sums over a column's rows run in another order than in the kernel above: a token's result differs from its by roundings.
+// Within these kernels it does not depend on how the sequence was cut or on what else the step holds.
+//
+// Workspace, float32: [T, heads, 6, DP] with DP = 16 RPT >= d (k, u, w, a u, r in the lanes' order: row k at
+// (k % 16) RPT + k / 16; then v in its own order; rows from d on are nought and leave the state's padding nought), then the
+// raw outputs [T, heads * d].
+#define DS_PARTS 16
+#define DS_VECS 6
+
 template <typename T>
 __global__ __launch_bounds__(256) void delta_prepare_kernel(const T* __restrict__ proj, long long row, int c_r, int c_k, int c_v, int c_a,
                                                             int c_w1, const T* __restrict__ W2, const float* __restrict__ w0,
@@ -129,15 +138,15 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const T* __restrict_
   constexpr int TT = 8;  // tokens a block: a thread reads its row of W_2 once for all of them
   __shared__ float st[TT][DR_MAX_LORA];
   const int t0 = blockIdx.x * TT, tokens = min(TT, num_tokens - t0);
-  const int hd = heads * d, dp = rpt * DR_PARTS;
-  for (int i = threadIdx.x; i < tokens * lora; i += blockDim.x) {
+  const int hd = heads * d, dp = rpt * DS_PARTS;
+  for (int i = threadIdx.x; i < TT * lora; i += blockDim.x) {
     const int tt = i / lora, j = i % lora;
-    st[tt][j] = tanhf(to_float(proj[(size_t)(t0 + tt) * row + c_w1 + j]));
+    st[tt][j] = tt < tokens ? tanhf(to_float(proj[(size_t)(t0 + tt) * row + c_w1 + j])) : 0.f;
   }
   __syncthreads();
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < hd; c += gridDim.y * blockDim.x) {
     const int head = c / d, k = c % d;
-    const int place = (k % DR_PARTS) * rpt + k / DR_PARTS;  // where the lane that owns row k finds it
+    const int place = (k % DS_PARTS) * rpt + k / DS_PARTS;  // where the lane that owns row k finds it
     float z[TT];
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) z[tt] = w0[c];
@@ -149,131 +158,136 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const T* __restrict_
     }
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
-      if (tt >= tokens) break;
-      const T* p = proj + (size_t)(t0 + tt) * row;
-      float* o = ws + ((size_t)(t0 + tt) * heads + head) * 5 * dp;
-      o[place] = to_float(p[c_k + c]);
-      o[dp + place] = to_float(p[c_r + c]);
-      o[2 * dp + place] = expf(-decay_coef * dr_sigmoid(z[tt]));
-      o[3 * dp + place] = dr_sigmoid(to_float(p[c_a + c]) + a_bias[c]);
-      o[4 * dp + k] = to_float(p[c_v + c]);
+      if (tt < tokens) {
+        const T* p = proj + (size_t)(t0 + tt) * row;
+        float* o = ws + ((size_t)(t0 + tt) * heads + head) * DS_VECS * dp;
+        o[place] = to_float(p[c_k + c]);
+        o[2 * dp + place] = expf(-decay_coef * dr_sigmoid(z[tt]));
+        o[3 * dp + place] = dr_sigmoid(to_float(p[c_a + c]) + a_bias[c]);
+        o[4 * dp + place] = to_float(p[c_r + c]);
+        o[5 * dp + k] = to_float(p[c_v + c]);
+      }
     }
   }
 }
 
-// Rows from d on of the workspace's vectors: nought (once a step, before the prepare kernel fills the rest).
+// Rows from d on of the workspace's vectors: nought (once a step, before the other kernels fill the rest).
 __global__ __launch_bounds__(256) void delta_pad_kernel(float* __restrict__ ws, long long units, int d, int rpt) {
-  const int dp = rpt * DR_PARTS, pad = dp - d;
-  const long long n = units * 5 * pad;
+  const int dp = rpt * DS_PARTS, pad = dp - d;
+  const long long n = units * DS_VECS * pad;
   for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
     const long long vec = i / pad;
     const int k = d + (int)(i % pad);
-    const int place = vec % 5 == 4 ? k : (k % DR_PARTS) * rpt + k / DR_PARTS;
+    const int place = vec % DS_VECS == 5 ? k : (k % DS_PARTS) * rpt + k / DS_PARTS;
     ws[vec * dp + place] = 0.f;
   }
 }
 
+// Grid (tokens, heads), a wave each: u = k / sqrt(sum(k^2) + 1e-6) and a u (in a's place).
+__global__ __launch_bounds__(64) void delta_unit_kernel(float* __restrict__ ws, int heads, int rpt) {
+  const int dp = rpt * DS_PARTS;
+  float* p = ws + ((size_t)blockIdx.x * heads + blockIdx.y) * DS_VECS * dp;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < dp; i += 64) ss = fmaf(p[i], p[i], ss);  // (the padding adds nought)
+  const float inv = 1.f / sqrtf(wave_sum(ss) + 1e-6f);
+  for (int i = threadIdx.x; i < dp; i += 64) {
+    const float u = p[i] * inv;
+    p[dp + i] = u;
+    p[3 * dp + i] *= u;
+  }
+}
+
 template <int RPT>
-struct DeltaVectors {
-  float k[RPT], r[RPT], w[RPT], a[RPT], v;
+struct DeltaRows {
+  float k[RPT], u[RPT], w[RPT], au[RPT], r[RPT], v;
 };
 
 template <int RPT>
-__device__ __forceinline__ void delta_fetch(DeltaVectors<RPT>& x, const float* __restrict__ p, int part, int v) {
-  constexpr int DP = RPT * DR_PARTS;
-  const float4* k4 = reinterpret_cast<const float4*>(p + part * RPT);
-  const float4* r4 = reinterpret_cast<const float4*>(p + DP + part * RPT);
-  const float4* w4 = reinterpret_cast<const float4*>(p + 2 * DP + part * RPT);
-  const float4* a4 = reinterpret_cast<const float4*>(p + 3 * DP + part * RPT);
+__device__ __forceinline__ void delta_fetch(DeltaRows<RPT>& x, const float* __restrict__ p, int part, int v) {
+  constexpr int DP = RPT * DS_PARTS;
+  float* dst[5] = {x.k, x.u, x.w, x.au, x.r};
 #pragma unroll
-  for (int q = 0; q < RPT / 4; ++q) {
-    const float4 a = k4[q], b = r4[q], c = w4[q], e = a4[q];
-    x.k[4 * q] = a.x, x.k[4 * q + 1] = a.y, x.k[4 * q + 2] = a.z, x.k[4 * q + 3] = a.w;
-    x.r[4 * q] = b.x, x.r[4 * q + 1] = b.y, x.r[4 * q + 2] = b.z, x.r[4 * q + 3] = b.w;
-    x.w[4 * q] = c.x, x.w[4 * q + 1] = c.y, x.w[4 * q + 2] = c.z, x.w[4 * q + 3] = c.w;
-    x.a[4 * q] = e.x, x.a[4 * q + 1] = e.y, x.a[4 * q + 2] = e.z, x.a[4 * q + 3] = e.w;
+  for (int vec = 0; vec < 5; ++vec) {
+    const float4* src = reinterpret_cast<const float4*>(p + vec * DP + part * RPT);
+#pragma unroll
+    for (int q = 0; q < RPT / 4; ++q) {
+      const float4 a = src[q];
+      dst[vec][4 * q] = a.x, dst[vec][4 * q + 1] = a.y, dst[vec][4 * q + 2] = a.z, dst[vec][4 * q + 3] = a.w;
+    }
   }
-  x.v = p[4 * DP + v];
+  x.v = p[5 * DP + v];
 }
 
-// One token of the recurrence for a lane's rows of its column (the arithmetic of delta_rule_kernel, in its order).
+// The sum of a value over the 16 lanes of its row, in every lane of the row (the same bits in all of them: a rotation by 8,
+// one by 4, then the two exchanges inside a group of four add the same pairs in every lane).
+__device__ __forceinline__ float row16_sum(float x) {
+#define DS_DPP_ADD(CTRL) x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false))
+  DS_DPP_ADD(0x128);  // row_ror:8
+  DS_DPP_ADD(0x124);  // row_ror:4
+  DS_DPP_ADD(0x4e);   // quad_perm:[2,3,0,1]
+  DS_DPP_ADD(0xb1);   // quad_perm:[1,0,3,2]
+#undef DS_DPP_ADD
+  return x;
+}
+
+// One token of the recurrence for a lane's rows of its column.
 template <int RPT>
-__device__ __forceinline__ float delta_token(float (&S)[RPT], const DeltaVectors<RPT>& x) {
-  float ss = 0.f;
-#pragma unroll
-  for (int j = 0; j < RPT; ++j) ss = fmaf(x.k[j], x.k[j], ss);
-  ss += __shfl_xor(ss, 1, ME_WAVE);
-  ss += __shfl_xor(ss, 2, ME_WAVE);
-  const float inv = 1.f / sqrtf(ss + 1e-6f);
+__device__ __forceinline__ float delta_token(float (&S)[RPT], const DeltaRows<RPT>& x) {
   float dot = 0.f;
 #pragma unroll
-  for (int j = 0; j < RPT; ++j) dot = fmaf(x.k[j] * inv, S[j], dot);
-  dot += __shfl_xor(dot, 1, ME_WAVE);
-  dot += __shfl_xor(dot, 2, ME_WAVE);
+  for (int j = 0; j < RPT; ++j) dot = fmaf(x.u[j], S[j], dot);
+  dot = row16_sum(dot);
   float o = 0.f;
 #pragma unroll
   for (int j = 0; j < RPT; ++j) {
-    const float u = x.k[j] * inv;
-    S[j] = fmaf(x.k[j], x.v, fmaf(x.w[j], S[j], -(x.a[j] * u) * dot));
+    S[j] = fmaf(x.k[j], x.v, fmaf(x.w[j], S[j], -x.au[j] * dot));
     o = fmaf(S[j], x.r[j], o);
   }
-  o += __shfl_xor(o, 1, ME_WAVE);
-  o += __shfl_xor(o, 2, ME_WAVE);
-  return o;
+  return row16_sum(o);
 }
 
-template <int RPT, bool AHEAD>
+template <int RPT, int AHEAD>
 __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict__ ws, float* __restrict__ state,
                                                         const int* __restrict__ item_start, const int* __restrict__ state_slots,
                                                         float* __restrict__ raw, int heads, int d) {
-  constexpr int DP = RPT * DR_PARTS;
+  constexpr int DP = RPT * DS_PARTS;
   const int item = blockIdx.x, head = blockIdx.y;
   const int slot = state_slots[item];
   if (slot < 0) return;
-  const int lane = threadIdx.x, v = blockIdx.z * 16 + lane / DR_PARTS, part = lane % DR_PARTS;
+  const int lane = threadIdx.x, v = blockIdx.z * 4 + lane / DS_PARTS, part = lane % DS_PARTS;
   const bool column = v < d;
   const int vv = column ? v : 0;  // (a lane beyond the head's columns reads a real one and writes none)
   float S[RPT];
   float* srow = state + ((size_t)slot * heads + head) * d * d;
 #pragma unroll
   for (int j = 0; j < RPT; ++j) {
-    const int k = part + DR_PARTS * j;
+    const int k = part + DS_PARTS * j;
     S[j] = column && k < d ? srow[(size_t)k * d + v] : 0.f;
   }
   const int first = item_start[item], last = item_start[item + 1];
-  const size_t step = (size_t)heads * 5 * DP;
-  const float* p = ws + ((size_t)first * heads + head) * 5 * DP;
-  float* out = raw + (size_t)first * heads * d + (size_t)head * d + v;
+  const size_t step = (size_t)heads * DS_VECS * DP, hd = (size_t)heads * d;
+  const float* p = ws + ((size_t)first * heads + head) * DS_VECS * DP;
+  float* out = raw + (size_t)first * hd + (size_t)head * d + v;
   const bool writes = column && part == 0;
-  if (AHEAD) {
-    DeltaVectors<RPT> x, y;
-    if (first < last) delta_fetch<RPT>(x, p, part, vv);
-    int t = first;
-    for (; t + 1 < last; t += 2) {  // two tokens a turn: each one's vectors arrive while the other is multiplied
-      delta_fetch<RPT>(y, p + step, part, vv);
-      const float o0 = delta_token<RPT>(S, x);
-      if (writes) out[0] = o0;
-      if (t + 2 < last) delta_fetch<RPT>(x, p + 2 * step, part, vv);
-      const float o1 = delta_token<RPT>(S, y);
-      if (writes) out[(size_t)heads * d] = o1;
-      p += 2 * step;
-      out += 2 * (size_t)heads * d;
+  DeltaRows<RPT> x[AHEAD];
+#pragma unroll
+  for (int b = 0; b < AHEAD; ++b)
+    if (first + b < last) delta_fetch<RPT>(x[b], p + b * step, part, vv);
+  for (int t = first; t < last; t += AHEAD) {  // AHEAD tokens a turn: a token's vectors arrive while those before it are multiplied
+#pragma unroll
+    for (int b = 0; b < AHEAD; ++b) {
+      if (t + b < last) {
+        const float o = delta_token<RPT>(S, x[b]);
+        if (writes) out[b * hd] = o;
+        if (t + b + AHEAD < last) delta_fetch<RPT>(x[b], p + (size_t)(b + AHEAD) * step, part, vv);
+      }
     }
-    if (t < last) {
-      const float o0 = delta_token<RPT>(S, x);
-      if (writes) out[0] = o0;
-    }
-  } else {
-    for (int t = first; t < last; ++t, p += step, out += (size_t)heads * d) {
-      DeltaVectors<RPT> x;
-      delta_fetch<RPT>(x, p, part, vv);
-      const float o = delta_token<RPT>(S, x);
-      if (writes) out[0] = o;
-    }
+    p += AHEAD * step;
+    out += AHEAD * hd;
   }
 #pragma unroll
   for (int j = 0; j < RPT; ++j) {
-    const int k = part + DR_PARTS * j;
+    const int k = part + DS_PARTS * j;
     if (column && k < d) srow[(size_t)k * d + v] = S[j];
   }
 }
@@ -294,13 +308,13 @@ __global__ __launch_bounds__(64) void delta_finish_kernel(const float* __restric
   for (int v = threadIdx.x; v < d; v += 64) y[v] = from_float<T>(o[v] * inv * norm_w[hc + v] * dr_sigmoid(to_float(p[v])) * out_scale);
 }
 
-static int delta_rows_per_lane(int d) { return d <= 64 ? 16 : d <= 128 ? 32 : 64; }
+static int delta_rows_per_lane(int d) { return 4 * ((d + 4 * DS_PARTS - 1) / (4 * DS_PARTS)); }  // 4, 8, 12 or 16
 
 // Bytes of workspace that me_delta_rule_steps needs for a step of `tokens` tokens.
 extern "C" long long me_delta_rule_workspace(long long tokens, int heads, int d) {
   if (tokens <= 0 || heads <= 0 || d <= 0 || d > DR_MAX_D) return 0;
-  const long long dp = (long long)delta_rows_per_lane(d) * DR_PARTS;
-  return (tokens * heads * 5 * dp + tokens * heads * d) * 4 + 256;
+  const long long dp = (long long)delta_rows_per_lane(d) * DS_PARTS;
+  return (tokens * heads * DS_VECS * dp + tokens * heads * d) * 4 + 256;
 }
 
 // proj [T, row]: the columns c_r, c_k, c_v, c_g, c_a (heads * d wide each) and c_w1 (`lora` wide). W2 [heads * d, lora] in the
@@ -362,32 +376,40 @@ extern "C" int me_delta_rule_steps(const void* proj, long long row, int c_r, int
     return me_fail("me_delta_rule_steps: the decay's inner projection at column %d of a row of %lld", c_w1, row);
   if (out_col < 0 || out_col + hd > out_row) return me_fail("me_delta_rule_steps: the result at column %d of a row of %lld", out_col, out_row);
   if (!workspace || ((uintptr_t)workspace & 15)) return me_fail("me_delta_rule_steps: a workspace at a multiple of 16 bytes");
-  const int rpt = delta_rows_per_lane(d), dp = rpt * DR_PARTS;
+  const int rpt = delta_rows_per_lane(d), dp = rpt * DS_PARTS;
   float* ws = (float*)workspace;
-  float* raw = ws + (size_t)num_tokens * heads * 5 * dp;
+  float* raw = ws + (size_t)num_tokens * heads * DS_VECS * dp;
   if (dp > d) {
-    const long long n = (long long)num_tokens * heads * 5 * (dp - d);
+    const long long n = (long long)num_tokens * heads * DS_VECS * (dp - d);
     delta_pad_kernel<<<(unsigned)std::min<long long>((n + 255) / 256, 4096), 256, 0, stream>>>(ws, (long long)num_tokens * heads, d, rpt);
   }
   const dim3 pgrid((num_tokens + 7) / 8, (unsigned)std::min<long long>((hd + 255) / 256, 64));
-  const dim3 sgrid(items, heads, (d + 15) / 16), fgrid(num_tokens, heads);
-#define DS_RUN(TT)                                                                                                              \
-  do {                                                                                                                          \
-    delta_prepare_kernel<TT><<<pgrid, 256, 0, stream>>>((const TT*)proj, row, c_r, c_k, c_v, c_a, c_w1, (const TT*)W2, w0, a_bias, \
-                                                        ws, num_tokens, heads, d, lora, rpt, decay_coef);                       \
-    if (rpt == 16)                                                                                                              \
-      delta_scan_kernel<16, true><<<sgrid, 64, 0, stream>>>(ws, state, item_start, state_slots, raw, heads, d);                 \
-    else if (rpt == 32)                                                                                                         \
-      delta_scan_kernel<32, false><<<sgrid, 64, 0, stream>>>(ws, state, item_start, state_slots, raw, heads, d);                \
-    else                                                                                                                        \
-      delta_scan_kernel<64, false><<<sgrid, 64, 0, stream>>>(ws, state, item_start, state_slots, raw, heads, d);                \
-    delta_finish_kernel<TT><<<fgrid, 64, 0, stream>>>(raw, (const TT*)proj, row, c_g, norm_w, (TT*)out, out_row, out_col,       \
-                                                      out_scale, heads, d, eps);                                               \
-  } while (0)
+  const dim3 sgrid(items, heads, (d + 3) / 4), tgrid(num_tokens, heads);
   if (dtype == ME_F32)
-    DS_RUN(float);
+    delta_prepare_kernel<float><<<pgrid, 256, 0, stream>>>((const float*)proj, row, c_r, c_k, c_v, c_a, c_w1, (const float*)W2, w0, a_bias,
+                                                           ws, num_tokens, heads, d, lora, rpt, decay_coef);
   else
-    DS_RUN(bf16_t);
-#undef DS_RUN
+    delta_prepare_kernel<bf16_t><<<pgrid, 256, 0, stream>>>((const bf16_t*)proj, row, c_r, c_k, c_v, c_a, c_w1, (const bf16_t*)W2, w0,
+                                                            a_bias, ws, num_tokens, heads, d, lora, rpt, decay_coef);
+  delta_unit_kernel<<<tgrid, 64, 0, stream>>>(ws, heads, rpt);
+  switch (rpt) {
+    case 4:
+      delta_scan_kernel<4, 4><<<sgrid, 64, 0, stream>>>(ws, state, item_start, state_slots, raw, heads, d);
+      break;
+    case 8:
+      delta_scan_kernel<8, 4><<<sgrid, 64, 0, stream>>>(ws, state, item_start, state_slots, raw, heads, d);
+      break;
+    case 12:
+      delta_scan_kernel<12, 2><<<sgrid, 64, 0, stream>>>(ws, state, item_start, state_slots, raw, heads, d);
+      break;
+    default:
+      delta_scan_kernel<16, 2><<<sgrid, 64, 0, stream>>>(ws, state, item_start, state_slots, raw, heads, d);
+  }
+  if (dtype == ME_F32)
+    delta_finish_kernel<float><<<tgrid, 64, 0, stream>>>(raw, (const float*)proj, row, c_g, norm_w, (float*)out, out_row, out_col, out_scale,
+                                                         heads, d, eps);
+  else
+    delta_finish_kernel<bf16_t><<<tgrid, 64, 0, stream>>>(raw, (const bf16_t*)proj, row, c_g, norm_w, (bf16_t*)out, out_row, out_col,
+                                                          out_scale, heads, d, eps);
   return me_check_launch("me_delta_rule_steps");
 }

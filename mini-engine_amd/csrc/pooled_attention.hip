@@ -66,13 +66,15 @@ __global__ __launch_bounds__(256) void pool_blocks_kernel(const T* __restrict__ 
   for (int e = threadIdx.x; e < d + dv; e += blockDim.x) {
     float sum = 0.f;
     if (e < d) {
-      for (int j = 0; j < pool; ++j) {
+#pragma unroll 8
+      for (int j = 0; j < pool; ++j) {  // (unrolled: the loads of eight keys are on their way together)
         const int key = first + j;
         sum += to_float(k_cache[(((size_t)table[key / bs] * nkv + kvh) * bs + key % bs) * d + e]);
       }
       k_pool[(((size_t)to_page * nkv + kvh) * bs + to_slot) * d + e] = from_float<T>(sum * inv);
     } else {
       const int ev = e - d;
+#pragma unroll 8
       for (int j = 0; j < pool; ++j) {
         const int key = first + j;
         sum += to_float(v_cache[(((size_t)table[key / bs] * nkv + kvh) * dv + ev) * bs + key % bs]);
