@@ -59,7 +59,8 @@ __global__ __launch_bounds__(RPT * DR_PARTS * 4) void delta_rule_kernel(
       sa[tid] = dr_sigmoid(to_float(p[c_a + c]) + a_bias[c]);
       float z = w0[c];
       const T* w2 = W2 + (size_t)c * lora;
-      for (int j = 0; j < lora; ++j) z = fmaf(to_float(w2[j]), st[j], z);
+#pragma unroll 8
+      for (int j = 0; j < lora; ++j) z = fmaf(to_float(w2[j]), st[j], z);  // (unrolled: eight loads on their way together)
       sw[tid] = expf(-decay_coef * dr_sigmoid(z));
     }
     __syncthreads();
@@ -393,8 +394,8 @@ extern "C" int me_delta_rule_steps(const void* proj, long long row, int c_r, int
                                                             a_bias, ws, num_tokens, heads, d, lora, rpt, decay_coef);
   delta_unit_kernel<<<tgrid, 64, 0, stream>>>(ws, heads, rpt);
   switch (rpt) {
-    case 4:
-      delta_scan_kernel<4, 4><<<sgrid, 64, 0, stream>>>(ws, state, item_start, state_slots, raw, heads, d);
+    case 4:  // (the further ahead a token's vectors are asked for, the less of their way from memory is waited for)
+      delta_scan_kernel<4, 8><<<sgrid, 64, 0, stream>>>(ws, state, item_start, state_slots, raw, heads, d);
       break;
     case 8:
       delta_scan_kernel<8, 4><<<sgrid, 64, 0, stream>>>(ws, state, item_start, state_slots, raw, heads, d);

@@ -23,6 +23,9 @@ __global__ __launch_bounds__(256) void whole_norm_scatter_kernel(
   const int t = blockIdx.x;
   const T* p = proj + (size_t)t * row;
   const int nq = nh * d, nk = nkv * d;
+  // (asked for ahead of the sums: the page's number is two trips to memory away)
+  const int pos = positions[t];
+  const int page = block_table[(size_t)token_item[t] * table_width + pos / bs], slot = pos % bs;
   float sq = 0.f, sk = 0.f;
   for (int i = threadIdx.x; i < nq; i += blockDim.x) {
     const float x = to_float(p[c_q + i]);
@@ -36,8 +39,6 @@ __global__ __launch_bounds__(256) void whole_norm_scatter_kernel(
   const float rk = rsqrtf(block_sum(sk, red) / (float)nk + eps);
   T* qo = q_out + (size_t)t * nq;
   for (int i = threadIdx.x; i < nq; i += blockDim.x) qo[i] = from_float<T>(to_float(p[c_q + i]) * rq * q_w[i]);
-  const int pos = positions[t];
-  const int page = block_table[(size_t)token_item[t] * table_width + pos / bs], slot = pos % bs;
   for (int i = threadIdx.x; i < nk; i += blockDim.x) {
     const int kvh = i / d, e = i % d;
     k_cache[(((size_t)page * nkv + kvh) * bs + slot) * d + e] = from_float<T>(to_float(p[c_k + i]) * rk * k_w[i]);
@@ -49,38 +50,57 @@ __global__ __launch_bounds__(256) void whole_norm_scatter_kernel(
   }
 }
 
-// Grid (tokens, kv heads): the block of a token that completes no pooled block returns at once.
+// Grid (runs of POOL_TOKENS tokens, kv heads), 256 threads: a block looks at its tokens one after the other and skips those that
+// complete no pooled block (a block of the grid for every token cost a step of 2,048 tokens more in starting blocks that had
+// nothing to do than in the work). For the others it fetches the pooled block's keys and values 16 positions at a time into
+// LDS ((d + dv) * 64 bytes), all loads of a round on their way together, and adds them up there, a thread an element, in
+// ascending position.
+#define POOL_TOKENS 8
+#define POOL_ROUND 16
+#define POOL_MAX_ROW 512  // d + dv at most
 template <typename T>
 __global__ __launch_bounds__(256) void pool_blocks_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                                                           T* __restrict__ k_pool, T* __restrict__ v_pool,
                                                           const int* __restrict__ positions, const int* __restrict__ token_item,
                                                           const int* __restrict__ block_table, int table_width, int nkv, int d, int dv,
-                                                          int bs, int pool) {
-  const int t = blockIdx.x, kvh = blockIdx.y;
+                                                          int bs, int pool, int num_tokens) {
+  extern __shared__ float tile[];  // [POOL_ROUND][d + dv]
+  const int kvh = blockIdx.y, tid = threadIdx.x;
+  for (int t = blockIdx.x * POOL_TOKENS; t < min(num_tokens, (int)(blockIdx.x + 1) * POOL_TOKENS); ++t) {
   const int pos = positions[t];
-  if ((pos + 1) % pool) return;
-  const int b = pos / pool, first = b * pool;
+  if ((pos + 1) % pool) continue;  // (the same for every thread of the block)
+  const int b = pos / pool, first = b * pool, w = d + dv;
   const int* table = block_table + (size_t)token_item[t] * table_width;
+  float sum[POOL_MAX_ROW / 256] = {0.f, 0.f};
+  for (int j0 = 0; j0 < pool; j0 += POOL_ROUND) {
+    const int n = min(POOL_ROUND, pool - j0);
+    for (int i = tid; i < n * d; i += 256) {  // neighbouring threads: neighbouring elements of a key
+      const int j = i / d, e = i % d, key = first + j0 + j;
+      tile[j * w + e] = to_float(k_cache[(((size_t)table[key / bs] * nkv + kvh) * bs + key % bs) * d + e]);
+    }
+    for (int i = tid; i < n * dv; i += 256) {  // neighbouring threads: neighbouring slots of a value's element
+      const int ev = i / n, j = i % n, key = first + j0 + j;
+      tile[j * w + d + ev] = to_float(v_cache[(((size_t)table[key / bs] * nkv + kvh) * dv + ev) * bs + key % bs]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < POOL_MAX_ROW / 256; ++q) {
+      const int e = tid + 256 * q;
+      if (e < w)
+        for (int j = 0; j < n; ++j) sum[q] += tile[j * w + e];
+    }
+    __syncthreads();
+  }
   const int to_page = table[b / bs], to_slot = b % bs;
   const float inv = 1.f / (float)pool;
-  for (int e = threadIdx.x; e < d + dv; e += blockDim.x) {
-    float sum = 0.f;
-    if (e < d) {
-#pragma unroll 8
-      for (int j = 0; j < pool; ++j) {  // (unrolled: the loads of eight keys are on their way together)
-        const int key = first + j;
-        sum += to_float(k_cache[(((size_t)table[key / bs] * nkv + kvh) * bs + key % bs) * d + e]);
-      }
-      k_pool[(((size_t)to_page * nkv + kvh) * bs + to_slot) * d + e] = from_float<T>(sum * inv);
-    } else {
-      const int ev = e - d;
-#pragma unroll 8
-      for (int j = 0; j < pool; ++j) {
-        const int key = first + j;
-        sum += to_float(v_cache[(((size_t)table[key / bs] * nkv + kvh) * dv + ev) * bs + key % bs]);
-      }
-      v_pool[(((size_t)to_page * nkv + kvh) * dv + ev) * bs + to_slot] = from_float<T>(sum * inv);
-    }
+#pragma unroll
+  for (int q = 0; q < POOL_MAX_ROW / 256; ++q) {
+    const int e = tid + 256 * q;
+    if (e < d)
+      k_pool[(((size_t)to_page * nkv + kvh) * bs + to_slot) * d + e] = from_float<T>(sum[q] * inv);
+    else if (e < w)
+      v_pool[(((size_t)to_page * nkv + kvh) * dv + (e - d)) * bs + to_slot] = from_float<T>(sum[q] * inv);
+  }
   }
 }
 
@@ -99,15 +119,17 @@ extern "C" int me_whole_norm_scatter(const void* proj, long long row, int c_q, i
       (c_v >= 0 && c_v + (long long)nkv * dv > row))
     return me_fail("me_whole_norm_scatter: columns %d, %d, %d of a row of %lld", c_q, c_k, c_v, row);
   if (pool > 0 && (!k_pool || !v_pool)) return me_fail("me_whole_norm_scatter: pooled blocks need pages of their own");
+  if (pool > 0 && d + dv > POOL_MAX_ROW) return me_fail("me_whole_norm_scatter: pooled keys and values of %d + %d elements (at most %d)", d, dv, POOL_MAX_ROW);
 #define WN_RUN(TT)                                                                                                                \
   do {                                                                                                                            \
     whole_norm_scatter_kernel<TT><<<num_tokens, 256, 0, stream>>>((const TT*)proj, row, c_q, c_k, c_v, q_w, k_w, positions,        \
                                                                   token_item, block_table, table_width, (TT*)q_out, (TT*)k_cache, \
                                                                   (TT*)v_cache, nh, nkv, d, dv, bs, eps);                         \
     if (pool > 0)                                                                                                                 \
-      pool_blocks_kernel<TT><<<dim3(num_tokens, nkv), d + dv >= 256 ? 256 : 64 * ((d + dv + 63) / 64), 0, stream>>>(              \
+      pool_blocks_kernel<TT><<<dim3((num_tokens + POOL_TOKENS - 1) / POOL_TOKENS, nkv), 256,                                       \
+                               (size_t)POOL_ROUND * (d + dv) * sizeof(float), stream>>>(                                          \
           (const TT*)k_cache, (const TT*)v_cache, (TT*)k_pool, (TT*)v_pool, positions, token_item, block_table, table_width, nkv, \
-          d, dv, bs, pool);                                                                                                       \
+          d, dv, bs, pool, num_tokens);                                                                                                       \
   } while (0)
   if (dtype == ME_F32)
     WN_RUN(float);
