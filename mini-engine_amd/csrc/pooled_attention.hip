@@ -14,6 +14,8 @@
 // Layouts: keys K[page, kv_head, slot, d]; values transposed V[page, kv_head, dv, slot]; pooled pages alike.
 #include "common.h"
 
+#define WN_Q_HELD 16
+#define WN_K_HELD 8
 template <typename T>
 __global__ __launch_bounds__(256) void whole_norm_scatter_kernel(
     const T* __restrict__ proj, long long row, int c_q, int c_k, int c_v, const float* __restrict__ q_w, const float* __restrict__ k_w,
@@ -26,6 +28,55 @@ __global__ __launch_bounds__(256) void whole_norm_scatter_kernel(
   // (asked for ahead of the sums: the page's number is two trips to memory away)
   const int pos = positions[t];
   const int page = block_table[(size_t)token_item[t] * table_width + pos / bs], slot = pos % bs;
+  if (nq <= WN_Q_HELD * 256 && nk <= WN_K_HELD * 256 && (c_v < 0 || dv == d)) {
+    // Rows that the block's registers hold (queries of up to 4,096 elements, keys of up to 2,048): the row and the weights are
+    // asked for once, together, and the block waits for memory twice (loads, then the two sums as one exchange), not five times.
+    float qv[WN_Q_HELD], qw[WN_Q_HELD], kv[WN_K_HELD], kw[WN_K_HELD], vv[WN_K_HELD];
+    float sq = 0.f, sk = 0.f;
+#pragma unroll
+    for (int n = 0; n < WN_Q_HELD; ++n) {
+      const int i = threadIdx.x + 256 * n;
+      qv[n] = i < nq ? to_float(p[c_q + i]) : 0.f;
+      qw[n] = i < nq ? q_w[i] : 0.f;
+    }
+#pragma unroll
+    for (int n = 0; n < WN_K_HELD; ++n) {
+      const int i = threadIdx.x + 256 * n;
+      kv[n] = i < nk ? to_float(p[c_k + i]) : 0.f;
+      kw[n] = i < nk ? k_w[i] : 0.f;
+      vv[n] = c_v >= 0 && i < nk ? to_float(p[c_v + i]) : kv[n];  // the values: a column of their own, or the keys as projected
+    }
+#pragma unroll
+    for (int n = 0; n < WN_Q_HELD; ++n) sq = fmaf(qv[n], qv[n], sq);
+#pragma unroll
+    for (int n = 0; n < WN_K_HELD; ++n) sk = fmaf(kv[n], kv[n], sk);
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    const int lane = threadIdx.x & (ME_WAVE - 1), wave = threadIdx.x / ME_WAVE;
+    if (lane == 0) {
+      red[wave] = sq;
+      red[4 + wave] = sk;
+    }
+    __syncthreads();
+    const float rq = rsqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)nq + eps);
+    const float rk = rsqrtf(((red[4] + red[5]) + (red[6] + red[7])) / (float)nk + eps);
+    T* qo = q_out + (size_t)t * nq;
+#pragma unroll
+    for (int n = 0; n < WN_Q_HELD; ++n) {
+      const int i = threadIdx.x + 256 * n;
+      if (i < nq) qo[i] = from_float<T>(qv[n] * rq * qw[n]);
+    }
+#pragma unroll
+    for (int n = 0; n < WN_K_HELD; ++n) {
+      const int i = threadIdx.x + 256 * n;
+      if (i < nk) {
+        const int kvh = i / d, e = i % d;
+        k_cache[(((size_t)page * nkv + kvh) * bs + slot) * d + e] = from_float<T>(kv[n] * rk * kw[n]);
+        v_cache[(((size_t)page * nkv + kvh) * dv + e) * bs + slot] = from_float<T>(vv[n]);
+      }
+    }
+    return;
+  }
   float sq = 0.f, sk = 0.f;
   for (int i = threadIdx.x; i < nq; i += blockDim.x) {
     const float x = to_float(p[c_q + i]);
