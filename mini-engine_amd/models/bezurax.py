@@ -55,6 +55,19 @@ def _need(d: dict, keys: tuple[str, ...], where: str) -> None:
         raise ValueError(f"{where} lacks required keys: {', '.join(missing)}")
 
 
+def owner_of(layers, i: int) -> int:
+    """The layer whose tensors layer i runs: itself, or the layer that its ``weights_of`` names (followed on if that one names
+    another in turn)."""
+    seen = {i}
+    j = i
+    while isinstance(layers[j], dict) and layers[j].get("weights_of") is not None:
+        j = int(layers[j]["weights_of"])
+        if not 0 <= j < len(layers) or j in seen:
+            raise ValueError(f"config.json layers[{i}]: weights_of must lead to a layer that has tensors of its own, not to {j}")
+        seen.add(j)
+    return j
+
+
 def _check_layer(layer: dict, where: str) -> None:
     _need(layer, ("type", "mixer"), where)
     if layer["type"] != "parallel":
@@ -109,9 +122,7 @@ class BezuraxConfig:
         for i, layer in enumerate(layers):
             where = f"config.json layers[{i}]"
             _check_layer(layer, where)
-            j = layer.get("weights_of")
-            if j is not None and (not 0 <= int(j) < len(layers) or layers[int(j)].get("weights_of") is not None):
-                raise ValueError(f"{where}: weights_of={j} must name a layer that has tensors of its own")
+            owner_of(layers, i)
         if eos is None:
             eos = cfg.get("eos_token_id")
         eos_ids = () if eos is None else ((int(eos),) if isinstance(eos, int) else tuple(int(e) for e in eos))
@@ -129,7 +140,11 @@ class BezuraxConfig:
         header = read_folder_header(folder)
         layers = []
         for i, layer in enumerate(cfg.get("layers", [])):
-            entry = header.get(f"l{int(layer.get('weights_of', i)) if isinstance(layer, dict) and layer.get('weights_of') is not None else i}.mix.right.w1")
+            try:
+                owner = owner_of(cfg["layers"], i)
+            except (ValueError, TypeError):
+                owner = i  # (from_dict says what is wrong with it)
+            entry = header.get(f"l{owner}.mix.right.w1")
             if entry is not None and isinstance(layer, dict) and isinstance(layer.get("mixer"), dict) and isinstance(layer["mixer"].get("right"), dict):
                 layer = dict(layer, mixer=dict(layer["mixer"], right=dict(layer["mixer"]["right"], decay_rank=int(entry.shape[0]))))
             layers.append(layer)
@@ -182,7 +197,7 @@ def plan_from_config(cfg: BezuraxConfig) -> ModelPlan:
             mixer_prefix=f"l{i}.mix", ffn_prefix=f"l{i}.mlp", mixer_norm_name=f"l{i}.norm1", ffn_norm_name=f"l{i}.norm2",
             arrangement="parallel", residual_scale=1.0))
     # a layer that runs another's weights is a second run of that layer, with a cache and state of its own
-    order = tuple(owners.index(i if layer.get("weights_of") is None else int(layer["weights_of"])) for i, layer in enumerate(cfg.layers))
+    order = tuple(owners.index(owner_of(cfg.layers, i)) for i in range(len(cfg.layers)))
     return ModelPlan(
         architecture=ARCHITECTURE, vocab_size=cfg.vocab, hidden_size=cfg.width, layers=tuple(layers), order=order, final_norm=norm,
         embed_name="embed", final_norm_name="final.norm", head_name="head", tie_word_embeddings=True,

@@ -92,6 +92,12 @@ def test_plan_takes_every_size_and_constant_from_the_config():
     pb = plan_from_config(BezuraxConfig.from_dict(bh.configs()["B"]))
     assert pb.layers[1].ffn is None and pb.layers[1].ffn_norm is None and pb.order == (0, 1, 1, 0)
     assert pb.final_norm.groups == 1 and pb.final_norm.eps == 1e-6
+    # a layer may name one that names another in turn, and a later one: all of them run the tensors of the one that has them
+    chain = dict(bh.configs()["B"])
+    b0, b1 = chain["layers"][0], chain["layers"][1]
+    chain["layers"] = [dict(b0, weights_of=3), dict(b1, weights_of=2), dict(b1, weights_of=3), b0]
+    pc = plan_from_config(BezuraxConfig.from_dict(chain))
+    assert len(pc.layers) == 1 and pc.order == (0, 0, 0, 0) and pc.layers[0].mixer_prefix == "l3.mix"
 
 
 def test_tensor_names_and_shapes():
