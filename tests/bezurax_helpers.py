@@ -43,12 +43,14 @@ def configs() -> dict[str, dict]:
     """Sizes, orders and constants that differ from one another in everything: one norm group and several; as many key/value
     heads as heads, and one; windows shorter than a page and longer than most prompts; pooled blocks of one key, of a page, of
     sizes that divide no page; groups of one expert, one group of all; every expert picked; layers without a feed-forward,
-    without a shared expert, and layers that run an earlier layer's weights; head sizes that are no multiple of 8."""
+    without a shared expert, and layers that run an earlier or a later layer's weights; head sizes that are no multiple of 8."""
     a0 = layer(left(4, 2, 24, 0.2, 40, 5), right(2, 16, 8), 0.7, 1.2, moe(6, 2, 40, 1.2, 3, 2, 1.5, shared=(24, 0.8)))
     a1 = layer(left(2, 1, 32, 0.15, 17, 3), right(3, 24, 12), 1.1, 0.6, moe(4, 3, 32, 2.0, 1, 1, 1.0))
     b0 = layer(left(6, 6, 20, 0.22, 64, 16), right(1, 40, 20), 1.0, 1.0, moe(8, 1, 48, 0.9, 8, 3, 2.5, shared=(72, 1.5)))
     b1 = layer(left(3, 1, 16, 0.3, 9, 1), right(4, 12, 4), 0.5, 1.5)
     c0 = layer(left(5, 1, 12, 0.3, 33, 7), right(2, 28, 16), 0.9, 0.9, moe(4, 4, 24, 1.0, 2, 2, 1.0, shared=(8, 3.0)))
+    e0 = layer(left(6, 2, 96, 0.1, 48, 10), right(3, 32, 16), 0.9, 1.1, moe(8, 3, 48, 1.4, 4, 2, 2.0, shared=(40, 1.1)))
+    e1 = layer(left(4, 4, 32, 0.18, 20, 4), right(2, 48, 8), 1.2, 0.7, moe(6, 2, 32, 2.5, 2, 2, 1.0))
     d0 = layer(left(2, 2, 64, 0.125, 128, 32), right(2, 64, 32), 1.0, 0.8, moe(6, 2, 64, 1.5, 2, 1, 2.0, shared=(64, 1.0)))
     return {
         "A": model(300, 96, 1e-5, 3, 0.5, [a0, a1, dict(a0, weights_of=0)]),
@@ -57,10 +59,13 @@ def configs() -> dict[str, dict]:
         "C": model(131, 100, 1e-6, 5, 0.25, [c0, dict(c0, weights_of=0)]),
         # heads of 64 under a window of 128 keys and pooled blocks of two pages
         "D": model(260, 128, 1e-5, 2, 0.3, [d0, d0]),
+        # heads of 96 and 32, three to a key/value head, blocks of 10 under a window of 48 (neither divides a page), a later
+        # layer's weights run first
+        "E": model(400, 192, 1e-6, 4, 0.4, [dict(e0, weights_of=1), e0, e1]),
     }
 
 
-BLOCK_SIZES = {"A": 16, "B": 32, "C": 8, "D": 16}
+BLOCK_SIZES = {"A": 16, "B": 32, "C": 8, "D": 16, "E": 16}
 
 
 def wants_of(cfg: dict):

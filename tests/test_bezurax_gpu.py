@@ -342,7 +342,7 @@ def requests_for(cfg, seed, lengths=(1, 23, 97, 150, 61)):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_every_way_of_cutting_gives_the_plain_logits(folders, name, dtype):
     """Whole prompts; most of a prompt and its tail token by token (replayed graphs); portions down to two tokens; up to
     four live requests in a pool whose pages and state slots are used again: all against the plain implementation."""
