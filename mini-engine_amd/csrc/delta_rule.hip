@@ -127,7 +127,7 @@ __global__ __launch_bounds__(RPT * DR_PARTS * 4) void delta_rule_kernel(
 //
 // Workspace, float32: [T, heads, 6, DP] with DP = 16 RPT >= d (k, u, w, a u, r in the lanes' order: row k at
 // (k % 16) RPT + k / 16; then v in its own order; rows from d on are nought and leave the state's padding nought), then the
-// raw outputs [T, heads * d].
+// raw outputs [T, heads, d rounded up to a multiple of 4].
 #define DS_PARTS 16
 #define DS_VECS 6
 
@@ -234,17 +234,23 @@ __device__ __forceinline__ float row16_sum(float x) {
 // One token of the recurrence for a lane's rows of its column.
 template <int RPT>
 __device__ __forceinline__ float delta_token(float (&S)[RPT], const DeltaRows<RPT>& x) {
-  float dot = 0.f;
+  // (two sums side by side, even rows and odd rows: a wave that walks the tokens alone waits for every result it needs next)
+  float dot0 = 0.f, dot1 = 0.f;
 #pragma unroll
-  for (int j = 0; j < RPT; ++j) dot = fmaf(x.u[j], S[j], dot);
-  dot = row16_sum(dot);
-  float o = 0.f;
-#pragma unroll
-  for (int j = 0; j < RPT; ++j) {
-    S[j] = fmaf(x.k[j], x.v, fmaf(x.w[j], S[j], -x.au[j] * dot));
-    o = fmaf(S[j], x.r[j], o);
+  for (int j = 0; j < RPT; j += 2) {
+    dot0 = fmaf(x.u[j], S[j], dot0);
+    dot1 = fmaf(x.u[j + 1], S[j + 1], dot1);
   }
-  return row16_sum(o);
+  const float dot = row16_sum(dot0 + dot1);
+  float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+  for (int j = 0; j < RPT; j += 2) {
+    S[j] = fmaf(x.k[j], x.v, fmaf(x.w[j], S[j], -x.au[j] * dot));
+    S[j + 1] = fmaf(x.k[j + 1], x.v, fmaf(x.w[j + 1], S[j + 1], -x.au[j + 1] * dot));
+    o0 = fmaf(S[j], x.r[j], o0);
+    o1 = fmaf(S[j + 1], x.r[j + 1], o1);
+  }
+  return row16_sum(o0 + o1);
 }
 
 template <int RPT, int AHEAD>
@@ -257,7 +263,7 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
   if (slot < 0) return;
   const int lane = threadIdx.x, v = blockIdx.z * 4 + lane / DS_PARTS, part = lane % DS_PARTS;
   const bool column = v < d;
-  const int vv = column ? v : 0;  // (a lane beyond the head's columns reads a real one and writes none)
+  const int vv = column ? v : 0;  // (a lane beyond the head's columns reads a real one; what it stores lands in the padding of the raw outputs)
   float S[RPT];
   float* srow = state + ((size_t)slot * heads + head) * d * d;
 #pragma unroll
@@ -266,26 +272,30 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
     S[j] = column && k < d ? srow[(size_t)k * d + v] : 0.f;
   }
   const int first = item_start[item], last = item_start[item + 1];
-  const size_t step = (size_t)heads * DS_VECS * DP, hd = (size_t)heads * d;
+  if (first >= last) return;
+  const int dpad = 4 * ((d + 3) / 4);  // the raw outputs' rows hold whole groups of four columns: every lane stores, no lane branches
+  const size_t step = (size_t)heads * DS_VECS * DP, hd = (size_t)heads * dpad;
   const float* p = ws + ((size_t)first * heads + head) * DS_VECS * DP;
-  float* out = raw + (size_t)first * hd + (size_t)head * d + v;
-  const bool writes = column && part == 0;
+  float* out = raw + (size_t)first * hd + (size_t)head * dpad + v;
   DeltaRows<RPT> x[AHEAD];
 #pragma unroll
-  for (int b = 0; b < AHEAD; ++b)
-    if (first + b < last) delta_fetch<RPT>(x[b], p + b * step, part, vv);
-  for (int t = first; t < last; t += AHEAD) {  // AHEAD tokens a turn: a token's vectors arrive while those before it are multiplied
+  for (int b = 0; b < AHEAD; ++b) delta_fetch<RPT>(x[b], p + (size_t)min(b, last - 1 - first) * step, part, vv);
+  // AHEAD tokens a turn, without a branch between them (a token's output is summed and stored while the next token's sums
+  // begin; the compiler moves instructions only inside a stretch without branches): a token's vectors are asked for AHEAD tokens
+  // ahead, those beyond the item's last token at the last token's place (fetched and not used).
+  int t = first;
+  for (; t + AHEAD <= last; t += AHEAD) {
 #pragma unroll
     for (int b = 0; b < AHEAD; ++b) {
-      if (t + b < last) {
-        const float o = delta_token<RPT>(S, x[b]);
-        if (writes) out[b * hd] = o;
-        if (t + b + AHEAD < last) delta_fetch<RPT>(x[b], p + (size_t)(b + AHEAD) * step, part, vv);
-      }
+      out[b * hd] = delta_token<RPT>(S, x[b]);  // (the 16 lanes of a column store the same number to the same place)
+      delta_fetch<RPT>(x[b], p + (size_t)min(b + AHEAD, last - 1 - t) * step, part, vv);
     }
     p += AHEAD * step;
     out += AHEAD * hd;
   }
+#pragma unroll
+  for (int b = 0; b < AHEAD; ++b)
+    if (t + b < last) out[b * hd] = delta_token<RPT>(S, x[b]);
 #pragma unroll
   for (int j = 0; j < RPT; ++j) {
     const int k = part + DS_PARTS * j;
@@ -299,7 +309,7 @@ __global__ __launch_bounds__(64) void delta_finish_kernel(const float* __restric
                                                           const float* __restrict__ norm_w, T* __restrict__ out, long long out_row,
                                                           int out_col, float out_scale, int heads, int d, float eps) {
   const int t = blockIdx.x, head = blockIdx.y, hc = head * d;
-  const float* o = raw + (size_t)t * heads * d + hc;
+  const float* o = raw + ((size_t)t * heads + head) * (4 * ((d + 3) / 4));
   float sq = 0.f;
   for (int v = threadIdx.x; v < d; v += 64) sq = fmaf(o[v], o[v], sq);
   sq = wave_sum(sq);
@@ -315,7 +325,7 @@ static int delta_rows_per_lane(int d) { return 4 * ((d + 4 * DS_PARTS - 1) / (4 
 extern "C" long long me_delta_rule_workspace(long long tokens, int heads, int d) {
   if (tokens <= 0 || heads <= 0 || d <= 0 || d > DR_MAX_D) return 0;
   const long long dp = (long long)delta_rows_per_lane(d) * DS_PARTS;
-  return (tokens * heads * DS_VECS * dp + tokens * heads * d) * 4 + 256;
+  return (tokens * heads * DS_VECS * dp + tokens * heads * (4 * ((d + 3) / 4))) * 4 + 256;
 }
 
 // proj [T, row]: the columns c_r, c_k, c_v, c_g, c_a (heads * d wide each) and c_w1 (`lora` wide). W2 [heads * d, lora] in the
