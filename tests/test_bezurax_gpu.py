@@ -141,7 +141,7 @@ def test_window_and_pooled_blocks_share_one_softmax(nh, nkv, d, window, pool, bs
             assert rel_err(cut[i], whole[i]) < 1e-6
 
 
-@pytest.mark.parametrize("nh,nkv,d,window,pool,bs", [(4, 2, 32, 40, 5, 16), (8, 1, 64, 100, 12, 16), (4, 4, 96, 96, 12, 64), (16, 8, 128, 256, 32, 16),
+@pytest.mark.parametrize("nh,nkv,d,window,pool,bs", [(4, 2, 32, 40, 5, 16), (8, 1, 64, 100, 12, 16), (6, 3, 96, 80, 10, 64), (16, 8, 128, 256, 32, 16),
                                                      (2, 1, 32, 1, 1, 16), (2, 2, 64, 700, 3, 32), (6, 2, 64, 64, 64, 64)])
 def test_the_matrix_core_kernels_see_what_the_general_kernel_sees(nh, nkv, d, window, pool, bs):
     """bfloat16 through the tiled kernel (prompts, portions, tokens beside portions) and the split-context kernel (steps of
