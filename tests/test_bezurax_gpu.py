@@ -146,14 +146,22 @@ def test_window_and_pooled_blocks_share_one_softmax(nh, nkv, d, window, pool, bs
 def test_the_matrix_core_kernels_see_what_the_general_kernel_sees(nh, nkv, d, window, pool, bs):
     """bfloat16 through the tiled kernel (prompts, portions, tokens beside portions) and the split-context kernel (steps of
     single tokens), into columns of wider rows: against the plain implementation, as close as the general kernel is."""
+    from mini_engine_amd.ops import kernels as K
+
     lens = [600, 77]
     rows, qw, kw, m, want, table, pages = pooled_case(nh, nkv, d, window, pool, bs, lens, torch.bfloat16, seed=nh + d + window)
-    whole = run_pooled(rows, qw, kw, m, table, pages, bs, torch.bfloat16, [[(0, 0, 600), (1, 0, 77)]], tiled=True)
-    cut = run_pooled(rows, qw, kw, m, table, pages, bs, torch.bfloat16, CUTS(599, 76) + [[(0, 599, 600), (1, 76, 77)]], tiled=True,
-                     out_cols=(nh * d + 32, 16, 0.7))
-    for i in (0, 1):
-        assert rel_err(whole[i], want[i]) < TOL[torch.bfloat16], i
-        assert rel_err(cut[i], want[i]) < TOL[torch.bfloat16], i
+    # the tiled kernel's blocks of 128 query columns, then those of 256 (which a step takes by its size: both are forced here)
+    for limits in ((1e30, 1e30), (0.0, 0.0)):
+        before = K.set_prefill_wide_limits(*limits)
+        try:
+            whole = run_pooled(rows, qw, kw, m, table, pages, bs, torch.bfloat16, [[(0, 0, 600), (1, 0, 77)]], tiled=True)
+            cut = run_pooled(rows, qw, kw, m, table, pages, bs, torch.bfloat16, CUTS(599, 76) + [[(0, 599, 600), (1, 76, 77)]], tiled=True,
+                             out_cols=(nh * d + 32, 16, 0.7))
+        finally:
+            K.set_prefill_wide_limits(*before)
+        for i in (0, 1):
+            assert rel_err(whole[i], want[i]) < TOL[torch.bfloat16], (i, limits)
+            assert rel_err(cut[i], want[i]) < TOL[torch.bfloat16], (i, limits)
 
 
 @pytest.mark.parametrize("tiled", [False, True])
