@@ -814,9 +814,10 @@ class Run {
     const int width = s_.lay.widths[g];
     const long long row = values_[op.in].cols, out_row = values_[op.out].cols;
     void* q = arena_.take((size_t)t_ * nh * d * elem_);
-    ok(me_whole_norm_scatter(bufs_[op.in], row, (int)op.i[8], (int)op.i[9], (int)op.i[10], (const float*)op.p[0], (const float*)op.p[1],
-                             idx(s_.lay.positions), idx(s_.lay.token_item), table, width, q, (void*)op.p[2], (void*)op.p[3],
-                             (void*)op.p[4], (void*)op.p[5], t_, nh, nkv, d, dv, bs, pool, op.f[0], dtype_, stream_));
+    ok(me_whole_norm_scatter_step(bufs_[op.in], row, (int)op.i[8], (int)op.i[9], (int)op.i[10], (const float*)op.p[0],
+                                  (const float*)op.p[1], idx(s_.lay.positions), idx(s_.lay.token_item), table, width, q, (void*)op.p[2],
+                                  (void*)op.p[3], (void*)op.p[4], (void*)op.p[5], t_, nh, nkv, d, dv, bs, pool, op.f[0],
+                                  s_.decode_only ? 1 : 0, dtype_, stream_));
     const float out_scale = op.f[2];  // (always given; nought is a scale like any other)
     if (pooled_takes_matrix_cores(op, dtype_, out_row) && s_.decode_only) {
       // one new token per item: the split-context kernel, which deals the pooled entries' tiles to its splits before the window's

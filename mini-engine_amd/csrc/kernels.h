@@ -183,6 +183,10 @@ int me_whole_norm_scatter(const void* proj, long long row, int c_q, int c_k, int
                           const int* positions, const int* token_item, const int* block_table, int table_width, void* q_out,
                           void* k_cache, void* v_cache, void* k_pool, void* v_pool, int num_tokens, int nh, int nkv, int d, int dv,
                           int bs, int pool, float eps, int dtype, hipStream_t stream);
+int me_whole_norm_scatter_step(const void* proj, long long row, int c_q, int c_k, int c_v, const float* q_w, const float* k_w,
+                          const int* positions, const int* token_item, const int* block_table, int table_width, void* q_out,
+                          void* k_cache, void* v_cache, void* k_pool, void* v_pool, int num_tokens, int nh, int nkv, int d, int dv,
+                          int bs, int pool, float eps, int single_tokens, int dtype, hipStream_t stream);
 int me_delta_rule(const void* proj, long long row, int c_r, int c_k, int c_v, int c_g, int c_a, int c_w1, const void* W2,
                   const float* w0, const float* a_bias, const float* norm_w, float* state, const int* item_start,
                   const int* state_slots, void* out, long long out_row, int out_col, float out_scale, int num_tokens, int items,

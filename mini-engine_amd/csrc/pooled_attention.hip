@@ -20,7 +20,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void whole_norm_scatter_kernel(
     const T* __restrict__ proj, long long row, int c_q, int c_k, int c_v, const float* __restrict__ q_w, const float* __restrict__ k_w,
     const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table, int table_width,
-    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int nh, int nkv, int d, int dv, int bs, float eps) {
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int nh, int nkv, int d, int dv, int bs, float eps,
+    T* __restrict__ k_pool, T* __restrict__ v_pool, int own_pool) {
   __shared__ float red[16];
   const int t = blockIdx.x;
   const T* p = proj + (size_t)t * row;
@@ -71,8 +72,29 @@ __global__ __launch_bounds__(256) void whole_norm_scatter_kernel(
       const int i = threadIdx.x + 256 * n;
       if (i < nk) {
         const int kvh = i / d, e = i % d;
-        k_cache[(((size_t)page * nkv + kvh) * bs + slot) * d + e] = from_float<T>(kv[n] * rk * kw[n]);
-        v_cache[(((size_t)page * nkv + kvh) * dv + e) * bs + slot] = from_float<T>(vv[n]);
+        const T key = from_float<T>(kv[n] * rk * kw[n]), value = from_float<T>(vv[n]);
+        k_cache[(((size_t)page * nkv + kvh) * bs + slot) * d + e] = key;
+        v_cache[(((size_t)page * nkv + kvh) * dv + e) * bs + slot] = value;
+        if (own_pool > 0 && (pos + 1) % own_pool == 0) {
+          // A step of single tokens (the host says so): the token that completes a pooled block adds up the block itself. The
+          // block's earlier keys came in earlier steps and lie in the pages; its own key is the last and is added last, as
+          // rounded: the sums are those of pool_blocks_kernel, in its order, and the launch of that kernel is saved.
+          const int b = pos / own_pool, first = b * own_pool;
+          const int* table = block_table + (size_t)token_item[t] * table_width;
+          float ks = 0.f, vs = 0.f;
+#pragma unroll 8
+          for (int j = 0; j < own_pool - 1; ++j) {
+            const int at = first + j, pg = table[at / bs], sl = at % bs;
+            ks += to_float(k_cache[(((size_t)pg * nkv + kvh) * bs + sl) * d + e]);
+            vs += to_float(v_cache[(((size_t)pg * nkv + kvh) * dv + e) * bs + sl]);
+          }
+          ks += to_float(key);
+          vs += to_float(value);
+          const int to_page = table[b / bs], to_slot = b % bs;
+          const float share = 1.f / (float)own_pool;
+          k_pool[(((size_t)to_page * nkv + kvh) * bs + to_slot) * d + e] = from_float<T>(ks * share);
+          v_pool[(((size_t)to_page * nkv + kvh) * dv + e) * bs + to_slot] = from_float<T>(vs * share);
+        }
       }
     }
     return;
@@ -158,10 +180,28 @@ __global__ __launch_bounds__(256) void pool_blocks_kernel(const T* __restrict__ 
 // proj [T, row]: queries at column c_q (nh * d), keys at c_k (nkv * d), values at c_v (nkv * dv; c_v < 0: the values are the
 // keys as projected, dv == d). q_w float32 [nh * d], k_w float32 [nkv * d]. pool > 0: the pooled pages get the blocks that
 // the step's tokens complete.
+extern "C" int me_whole_norm_scatter_step(const void* proj, long long row, int c_q, int c_k, int c_v, const float* q_w, const float* k_w,
+                                          const int* positions, const int* token_item, const int* block_table, int table_width,
+                                          void* q_out, void* k_cache, void* v_cache, void* k_pool, void* v_pool, int num_tokens, int nh,
+                                          int nkv, int d, int dv, int bs, int pool, float eps, int single_tokens, int dtype,
+                                          hipStream_t stream);
+
 extern "C" int me_whole_norm_scatter(const void* proj, long long row, int c_q, int c_k, int c_v, const float* q_w, const float* k_w,
                                      const int* positions, const int* token_item, const int* block_table, int table_width,
                                      void* q_out, void* k_cache, void* v_cache, void* k_pool, void* v_pool, int num_tokens, int nh,
                                      int nkv, int d, int dv, int bs, int pool, float eps, int dtype, hipStream_t stream) {
+  return me_whole_norm_scatter_step(proj, row, c_q, c_k, c_v, q_w, k_w, positions, token_item, block_table, table_width, q_out, k_cache,
+                                    v_cache, k_pool, v_pool, num_tokens, nh, nkv, d, dv, bs, pool, eps, 0, dtype, stream);
+}
+
+// As me_whole_norm_scatter; single_tokens != 0: every item of the step brings one token (every earlier position of a pooled block
+// then lies in the pages already), and the kernel that writes the pages adds up the pooled blocks itself where it holds the rows
+// in registers.
+extern "C" int me_whole_norm_scatter_step(const void* proj, long long row, int c_q, int c_k, int c_v, const float* q_w, const float* k_w,
+                                          const int* positions, const int* token_item, const int* block_table, int table_width,
+                                          void* q_out, void* k_cache, void* v_cache, void* k_pool, void* v_pool, int num_tokens, int nh,
+                                          int nkv, int d, int dv, int bs, int pool, float eps, int single_tokens, int dtype,
+                                          hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (nh <= 0 || nkv <= 0 || nkv > 65535 || d <= 0 || dv <= 0 || bs <= 0 || table_width <= 0 || pool < 0)
     return me_fail("me_whole_norm_scatter: nh=%d nkv=%d d=%d dv=%d bs=%d pool=%d", nh, nkv, d, dv, bs, pool);
@@ -171,12 +211,16 @@ extern "C" int me_whole_norm_scatter(const void* proj, long long row, int c_q, i
     return me_fail("me_whole_norm_scatter: columns %d, %d, %d of a row of %lld", c_q, c_k, c_v, row);
   if (pool > 0 && (!k_pool || !v_pool)) return me_fail("me_whole_norm_scatter: pooled blocks need pages of their own");
   if (pool > 0 && d + dv > POOL_MAX_ROW) return me_fail("me_whole_norm_scatter: pooled keys and values of %d + %d elements (at most %d)", d, dv, POOL_MAX_ROW);
+  // (the rows that the page-write kernel holds in registers: see its first branch)
+  const bool own_pool = single_tokens && pool > 0 && (long long)nh * d <= WN_Q_HELD * 256 && (long long)nkv * d <= WN_K_HELD * 256 &&
+                        (c_v < 0 || dv == d);
 #define WN_RUN(TT)                                                                                                                \
   do {                                                                                                                            \
     whole_norm_scatter_kernel<TT><<<num_tokens, 256, 0, stream>>>((const TT*)proj, row, c_q, c_k, c_v, q_w, k_w, positions,        \
                                                                   token_item, block_table, table_width, (TT*)q_out, (TT*)k_cache, \
-                                                                  (TT*)v_cache, nh, nkv, d, dv, bs, eps);                         \
-    if (pool > 0)                                                                                                                 \
+                                                                  (TT*)v_cache, nh, nkv, d, dv, bs, eps, (TT*)k_pool,             \
+                                                                  (TT*)v_pool, own_pool ? pool : 0);                              \
+    if (pool > 0 && !own_pool)                                                                                                    \
       pool_blocks_kernel<TT><<<dim3((num_tokens + POOL_TOKENS - 1) / POOL_TOKENS, nkv), 256,                                       \
                                (size_t)POOL_ROUND * (d + dv) * sizeof(float), stream>>>(                                          \
           (const TT*)k_cache, (const TT*)v_cache, (TT*)k_pool, (TT*)v_pool, positions, token_item, block_table, table_width, nkv, \

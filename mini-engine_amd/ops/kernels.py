@@ -1371,11 +1371,13 @@ def gemm_bf16_stream_norm_streams(xs: torch.Tensor, delta, rewrite: torch.Tensor
 # ------------------------------------------------------------------ attention over a window and pooled blocks
 def whole_norm_scatter(proj: torch.Tensor, q_w: torch.Tensor, k_w: torch.Tensor, positions, token_item, block_table, k_cache, v_cache,
                        nh: int, nkv: int, d: int, dv: int, eps: float, q_col: int = 0, k_col: int | None = None, v_col: int = -1,
-                       k_pool: torch.Tensor | None = None, v_pool: torch.Tensor | None = None, pooled_block: int = 0) -> torch.Tensor:
+                       k_pool: torch.Tensor | None = None, v_pool: torch.Tensor | None = None, pooled_block: int = 0,
+                       single_tokens: bool = False) -> torch.Tensor:
     """q and k of ``proj`` ``[T, row]`` (queries at column ``q_col``, keys at ``k_col``, default right behind the queries) normed over
     their whole projection with the float32 weights ``q_w`` ``[nh * d]`` and ``k_w`` ``[nkv * d]``; the normed keys go to the key pages,
     the values (the column ``v_col``; -1: the keys as projected) to the value pages; with ``pooled_block`` P the means of the blocks
-    of P keys and values that the step's tokens complete go to the pooled pages. Returns the normed queries ``[T, nh, d]``."""
+    of P keys and values that the step's tokens complete go to the pooled pages. ``single_tokens``: every item of the step brings
+    one token (the kernel that writes the pages then adds up the pooled blocks itself). Returns the normed queries ``[T, nh, d]``."""
     _want(proj, "proj", None, (None, None))
     t, row = proj.shape
     k_col = q_col + nh * d if k_col is None else k_col
@@ -1388,10 +1390,10 @@ def whole_norm_scatter(proj: torch.Tensor, q_w: torch.Tensor, k_w: torch.Tensor,
         _want(k_pool, "k_pool", proj.dtype, tuple(k_cache.shape))
         _want(v_pool, "v_pool", proj.dtype, tuple(v_cache.shape))
     q = torch.empty((t, nh, d), dtype=proj.dtype, device=proj.device)
-    check(lib().me_whole_norm_scatter(_p(proj), _i64(row), _i(q_col), _i(k_col), _i(v_col), _p(q_w), _p(k_w), _p(positions), _p(token_item),
-                                      _p(block_table), _i(block_table.shape[1]), _p(q), _p(k_cache), _p(v_cache), _p(k_pool), _p(v_pool),
-                                      _i(t), _i(nh), _i(nkv), _i(d), _i(dv), _i(bs), _i(pooled_block), _f(eps), _i(_code(proj.dtype)),
-                                      _stream()))
+    check(lib().me_whole_norm_scatter_step(_p(proj), _i64(row), _i(q_col), _i(k_col), _i(v_col), _p(q_w), _p(k_w), _p(positions),
+                                           _p(token_item), _p(block_table), _i(block_table.shape[1]), _p(q), _p(k_cache), _p(v_cache),
+                                           _p(k_pool), _p(v_pool), _i(t), _i(nh), _i(nkv), _i(d), _i(dv), _i(bs), _i(pooled_block), _f(eps),
+                                           _i(1 if single_tokens else 0), _i(_code(proj.dtype)), _stream()))
     return q
 
 

@@ -100,7 +100,7 @@ def run_pooled(rows, qw, kw, m, table, pages, bs, dtype, cuts, tiled, out_cols=N
         item = torch.tensor([n for n, (i, lo, hi) in enumerate(step) for _ in range(lo, hi)], dtype=torch.int32).cuda()
         tab = table[[i for i, lo, hi in step]].cuda().contiguous()
         q = K.whole_norm_scatter(proj, qw.cuda(), kw.cuda(), pos, item, tab, kc, vc, nh, nkv, d, d, 1e-5, k_pool=kp, v_pool=vp,
-                                 pooled_block=pool)
+                                 pooled_block=pool, single_tokens=all(hi - lo == 1 for i, lo, hi in step))
         row, col, scale = out_cols or (nh * d, 0, 1.0)
         out = torch.full((proj.shape[0], row), 7.0, dtype=dtype).cuda()
         if tiled:
