@@ -67,6 +67,23 @@ class YarnRotarySpec:
 
 
 @dataclass(frozen=True)
+class ScaledRotarySpec:
+    """Rotary encoding whose slow pairs are slowed for contexts beyond the ``original`` one. With ``f_j = theta ** (-2j / rotary_dim)``
+    and the wavelength ``l_j = 2 pi / f_j``: pairs with ``l_j < original / high`` turn at ``f_j``, pairs with ``l_j > original / low``
+    at ``f_j / factor``, and those between at ``(1 - s) f_j / factor + s f_j`` with ``s = (original / l_j - low) / (high - low)``.
+    Cosines and sines are not multiplied by anything. The table is worked out in double precision and rounded once."""
+
+    rotary_dim: int
+    theta: float
+    factor: float
+    low: float
+    high: float
+    original: float
+    kind: str = "scaled_rotary"
+    pairing: str = "halves"
+
+
+@dataclass(frozen=True)
 class AttentionSpec:
     """Causal grouped-query attention over a paged key/value cache.
 
@@ -112,6 +129,14 @@ class AttentionSpec:
     # the block's keys as the cache holds them and the mean of its values; tokens and blocks share one softmax. Tokens that have
     # left the window and whose block is not yet complete behind it are not seen
     pooled_block: int = 0
+    # with q and k normed over the whole projection: > 0, a short causal convolution over time of that many taps on every channel of
+    # q, k and v, directly behind the projections (``y_t = sum_j w[:, j] u_(t - taps + 1 + j)``, zeros before the sequence; weights
+    # ``[channels, taps]`` under the roles ``q_conv k_conv v_conv``); the last ``taps - 1`` projections of a sequence are its state
+    conv_taps: int = 0
+    # > 0: every scaled score s becomes softcap * tanh(s / softcap) before the softmax
+    softcap: float = 0.0
+    # one is added to the softmax's denominator: a sink whose score is 0 and which has no value
+    unit_sink: bool = False
 
     @property
     def v_dim(self) -> int:
@@ -150,12 +175,15 @@ class LatentAttentionSpec:
     output_gate: bool = False
     names: tuple[tuple[str, str], ...] = ()
     kind: str = "latent_attention"
+    # another layer (index into ``ModelPlan.layers``) whose latents and shared key parts this layer reads, as that layer's pages hold
+    # them; it has no latent projection of its own (no ``dkv``, no ``dkv_norm``), but maps, queries and gates of its own
+    cache_from: int | None = None
 
     @property
     def kv_elements_per_token(self) -> int:
         """Elements one token occupies in this layer's pages at most: the key ``[c | shared part]`` and its value rows (the
         latent once more; the whole key once more where the matrix-core kernels serve the layer)."""
-        return 2 * (self.latent_rank + self.rotary_dim)
+        return 0 if self.cache_from is not None else 2 * (self.latent_rank + self.rotary_dim)
 
 
 @dataclass(frozen=True)
@@ -216,6 +244,32 @@ class DeltaRuleSpec:
 
 
 @dataclass(frozen=True)
+class TimeMixSpec:
+    """Linear attention with a decay per token, head and key channel and a bonus for the current token, a ``head_dim x head_dim``
+    float32 state per request and head (zero at first). With h' the input of the token before (zeros for a sequence's first), each of r,
+    k, v, g, w reads its own blend ``h + (h' - h) * mu``; r, k, v are projections of theirs (``num_heads x head_dim``), ``gate =
+    silu(W_g blend_g)``, the decay ``w = exp(-exp(W_2 tanh(W_1 blend_w) + w_0))`` (inner size ``decay_rank``), and::
+
+        o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t,        S_t = diag(w_t) S_(t-1) + k_t v_t^T
+
+    Each head's o is divided by its root mean square (``norm_eps``); the heads together are multiplied by a weight and by the gate and go
+    through the output projection. The last token's input is part of the state. ``names`` maps the roles ``mu_r mu_k mu_v mu_g mu_w r k
+    v g w1 w2 w0 u norm o``."""
+
+    hidden_size: int
+    num_heads: int
+    head_dim: int
+    decay_rank: int
+    norm_eps: float
+    names: tuple[tuple[str, str], ...] = ()
+    kind: str = "time_mix"
+
+    @property
+    def state_elements(self) -> int:
+        return self.num_heads * self.head_dim * self.head_dim + self.hidden_size
+
+
+@dataclass(frozen=True)
 class PairMixerSpec:
     """Two mixers side by side that read the same input; the result is ``left_scale * left + right_scale * right``. Their tensors
     lie under ``<prefix>.<left_name>`` and ``<prefix>.<right_name>``; each keeps a cache or state of its own."""
@@ -246,6 +300,33 @@ class GatedMlpSpec:
 
 
 @dataclass(frozen=True)
+class ActivatedMlpSpec:
+    """Dense feed-forward without a gate: ``down(act(up(x)))`` without biases; ``activation`` is "relu2" (the square of relu),
+    "gelu_tanh" or "silu"."""
+
+    hidden_size: int
+    intermediate_size: int
+    activation: str = "relu2"
+    kind: str = "activated_mlp"
+    names: tuple[tuple[str, str], ...] = ()  # roles ``up down`` -> the checkpoint's suffixes
+
+
+@dataclass(frozen=True)
+class TokenInputSpec:
+    """An input that a layer takes from the token itself, behind its feed-forward: with e the elements ``[index * dim, (index + 1) *
+    dim)`` of the token's row of the table ``table_name`` ``[vocab, *]``, ``y = W_proj (act(W_gate x) * e)`` and ``x += y / sqrt(mean(y^2) +
+    eps) * w`` (an RMS norm with a plain weight). ``prefix`` names the tensors ``<prefix>.<gate|proj|norm>``."""
+
+    table_name: str
+    dim: int
+    index: int
+    eps: float
+    prefix: str
+    activation: str = "gelu_tanh"
+    names: tuple[tuple[str, str], ...] = ()  # roles ``gate proj norm``
+
+
+@dataclass(frozen=True)
 class RoutedExpertsSpec:
     """A feed-forward of ``num_experts`` gated feed-forwards of ``intermediate_size`` each, of which a token uses the ``top_k``
     with the largest router logits (float32), weighted by the softmax over those logits alone. Tensors: ``<prefix>.<router>``
@@ -273,6 +354,15 @@ class RoutedExpertsSpec:
     # uses, multiplied by the sigmoid of one number per token (``<prefix>.<shared>.<shared_gate>`` ``[1, hidden]``)
     shared_size: int = 0
     shared_limit: float = 0.0
+    # "softmax_all": scores are the softmax over all router outputs; the picks go by score + correction (a tensor under the role
+    # ``correction``, when ``score_correction``), the weights are the picks' scores as they are, times ``route_scale``. The last
+    # ``identity_experts`` router outputs (behind the ``num_experts`` with tensors) are identity experts: their result is the input
+    identity_experts: int = 0
+    score_correction: bool = False
+    # False: an expert is ``down(act(up x))`` with an activation of :class:`ActivatedMlpSpec` (no gate rows)
+    gated: bool = True
+    # False: nothing multiplies the shared expert's result (no tensor under the role ``shared_gate``)
+    shared_gated: bool = True
 
 
 @dataclass(frozen=True)
@@ -295,6 +385,9 @@ class LayerSpec:
     feed-forward has a norm of its own, of the same x: ``x += residual_scale * (mixer(norm1(x)) + ffn(norm2(x)))``.
     ``arrangement == "hyper_connections"``: as ``pre_norm`` over several residual streams: each part reads and rewrites them by
     its :class:`HyperConnectionSpec` (``mixer_streams``, ``ffn_streams``); ``ffn`` may be None.
+    ``arrangement == "result_norm"``: the norms sit on the sublayers' results, and the sublayers read the stream itself:
+    ``x += norm1(mixer(x)); x += norm2(ffn(x))``; ``ffn`` may be None. ``token_input`` (any arrangement that takes it): an input from
+    the token itself behind the feed-forward (:class:`TokenInputSpec`).
     The ``*_prefix`` / ``*_name`` strings are the checkpoint names of this layer's tensors.
     """
 
@@ -310,6 +403,7 @@ class LayerSpec:
     residual_scale: float = 1.0
     mixer_streams: Any | None = None
     ffn_streams: Any | None = None
+    token_input: Any | None = None
 
 
 @dataclass(frozen=True)
@@ -331,6 +425,7 @@ class ModelPlan:
     embedding_multiplier: float | None = None  # the looked-up rows are multiplied by it (None: as they are)
     logit_scale: float | None = None  # the logits are multiplied by it (None: as they are)
     residual_streams: int = 0  # > 0: that many residual streams, all the embedding at first, summed before the final norm
+    token_table_columns: int = 0  # > 0: the row length of the table that the layers' token inputs read slices of
 
     def __post_init__(self) -> None:
         n = len(self.layers)

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
     int table_width, T* __restrict__ out, int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
     const float* __restrict__ unturn, int un_pairing, float scale, int wpu, const float* __restrict__ sink,
     const T* __restrict__ gate, size_t gate_row, const T* __restrict__ k_pool, const T* __restrict__ v_pool, int pool,
-    long long out_row, int out_col, float out_scale) {
+    long long out_row, int out_col, float out_scale, float softcap) {
   constexpr int DMAX = KMAX * ME_WAVE;  // the largest head this instance takes
   __shared__ float qs[8][DMAX];
   __shared__ float parts[8][DMAX + 2];  // with several waves per unit: a round's results (values, maximum, sum)
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
         } else {
           for (int i = 0; i < d; ++i) dot = fmaf(qw[i], to_float(krow[i]), dot);
         }
-        s = dot;
+        s = softcap > 0.f ? softcap * tanhf(dot / softcap) : dot;  // (bounded scores: the scaled score through a tanh)
       }
       const float m_new = fmaxf(m, wave_max(s));  // at least one key of the tile is visible
       const float pr = valid ? expf(s - m_new) : 0.f;
@@ -469,12 +469,13 @@ __global__ __launch_bounds__(1024) void attention_shared_f32_kernel(
 // values at the positions b pool .. b pool + pool - 1) that are visible, beside the window's keys, once the window has passed
 // them wholly; they share the softmax with the window's keys. out_row, out_col: the result's rows are out_row elements apart
 // (0: nh * dv) and begin at column out_col; out_scale multiplies the result before it is rounded.
-extern "C" int me_attention_general_pooled(const void* q, const void* k_cache, const void* v_cache, const int* positions,
+// softcap > 0: every scaled score s becomes softcap * tanh(s / softcap) before the softmax.
+extern "C" int me_attention_general_capped(const void* q, const void* k_cache, const void* v_cache, const int* positions,
                                            const int* token_item, const int* block_table, int table_width, void* out,
                                            int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
                                            const float* unturn, int un_pairing, float scale, const float* sink, const void* gate,
                                            long long gate_row, const void* k_pool, const void* v_pool, int pool, long long out_row,
-                                           int out_col, float out_scale, int dtype, int items, hipStream_t stream) {
+                                           int out_col, float out_scale, float softcap, int dtype, int items, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (pool < 0 || (pool > 0 && (window <= 0 || keep_first > 0 || !k_pool || !v_pool)))
     return me_fail("me_attention_general: pooled blocks of %d keys need a window, pages of their own and no kept first keys", pool);
@@ -487,7 +488,7 @@ extern "C" int me_attention_general_pooled(const void* q, const void* k_cache, c
     return me_fail("me_attention_general: keep_first=%d needs a window", keep_first);
   if (unturn && (dv % 2 || (un_pairing & ~1))) return me_fail("me_attention_general: values of size %d, pairing %d", dv, un_pairing);
   const bool plain = dv == d && keep_first == 0 && !unturn && !sink && !gate && !big && pool == 0 && out_row <= 0 && out_col == 0 &&
-                     out_scale == 1.f;
+                     out_scale == 1.f && !(softcap > 0.f);
   if (nh <= 0 || nkv <= 0 || nh % nkv)
     return me_fail("me_attention_general: %d query heads are not a multiple of %d key/value heads", nh, nkv);
   if (bs <= 0 || table_width <= 0 || window < 0)
@@ -533,7 +534,7 @@ extern "C" int me_attention_general_pooled(const void* q, const void* k_cache, c
   attention_general_kernel<TT, KK><<<blocks, waves * 64, 0, stream>>>(                                                         \
       (const TT*)q, (const TT*)k_cache, (const TT*)v_cache, positions, token_item, block_table, table_width, (TT*)out, num_tokens, \
       nh, nkv, d, dv, bs, window, keep_first, unturn, un_pairing, scale, wpu, sink, (const TT*)gate, (size_t)gate_row,             \
-      (const TT*)k_pool, (const TT*)v_pool, pool, out_row > 0 ? out_row : (long long)nh * dv, out_col, out_scale)
+      (const TT*)k_pool, (const TT*)v_pool, pool, out_row > 0 ? out_row : (long long)nh * dv, out_col, out_scale, softcap)
   if (dtype == ME_F32) {
     if (big)
       ME_AG_LAUNCH(float, AG_MAX_D_WIDE / ME_WAVE);
@@ -547,6 +548,17 @@ extern "C" int me_attention_general_pooled(const void* q, const void* k_cache, c
   }
 #undef ME_AG_LAUNCH
   return me_check_launch("me_attention_general");
+}
+
+extern "C" int me_attention_general_pooled(const void* q, const void* k_cache, const void* v_cache, const int* positions,
+                                           const int* token_item, const int* block_table, int table_width, void* out,
+                                           int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
+                                           const float* unturn, int un_pairing, float scale, const float* sink, const void* gate,
+                                           long long gate_row, const void* k_pool, const void* v_pool, int pool, long long out_row,
+                                           int out_col, float out_scale, int dtype, int items, hipStream_t stream) {
+  return me_attention_general_capped(q, k_cache, v_cache, positions, token_item, block_table, table_width, out, num_tokens, nh, nkv,
+                                     d, dv, bs, window, keep_first, unturn, un_pairing, scale, sink, gate, gate_row, k_pool, v_pool,
+                                     pool, out_row, out_col, out_scale, 0.f, dtype, items, stream);
 }
 
 extern "C" int me_attention_general_gated(const void* q, const void* k_cache, const void* v_cache, const int* positions,

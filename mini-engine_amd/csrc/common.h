@@ -63,6 +63,10 @@ __device__ __forceinline__ me_u32x2 stream_load8(const void* p) {
 // ME_GATE_CLAMPED_SIGMOID (kernels that take a limit beside the code): g' = min(gate, limit), u' = clamp(up, -limit, limit),
 // g' sigmoid(1.702 g') (u' + 1).
 enum MeGate { ME_GATE_NONE = 0, ME_GATE_SILU = 1, ME_GATE_GELU_TANH = 2, ME_GATE_CLAMPED_SIGMOID = 3 };
+// Activations of a feed-forward without a gate, act(up): codes from 16 on, so that one argument says both which activation and
+// that the product has no gate rows. ME_ACT_RELU2: max(z, 0)^2.
+enum MeAct { ME_ACT_RELU2 = 16, ME_ACT_GELU_TANH = 17, ME_ACT_SILU = 18 };
+__host__ __device__ __forceinline__ bool act_is_ungated(int code) { return code >= 16; }
 
 __device__ __forceinline__ float gate_act(float g, int code) {
   if (code == ME_GATE_GELU_TANH) {  // 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
@@ -70,6 +74,13 @@ __device__ __forceinline__ float gate_act(float g, int code) {
     return 0.5f * g * (1.f + tanhf(u));
   }
   return g / (1.f + expf(-g));  // silu
+}
+// act(z) of an ungated feed-forward.
+__device__ __forceinline__ float ungated_act(float z, int code) {
+  if (code == ME_ACT_GELU_TANH) return gate_act(z, ME_GATE_GELU_TANH);
+  if (code == ME_ACT_SILU) return gate_act(z, ME_GATE_SILU);
+  const float r = fmaxf(z, 0.f);
+  return r * r;
 }
 // act(gate) * up for every code, the forms with a limit among them.
 __device__ __forceinline__ float gated_pair(float g, float u, int code, float limit) {

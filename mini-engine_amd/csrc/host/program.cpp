@@ -171,11 +171,13 @@ bool attention_takes_tiled_prefill(const Op& op, int dtype) {
 // one size that the kernels are built for, up to 16 heads to a key/value head, results at rows and a column that are multiples of 4.
 bool pooled_takes_matrix_cores(const Op& op, int dtype, long long out_row) {
   const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2], dv = (int)op.i[3], bs = (int)op.i[4];
+  if (op.p[9] || op.f[3] > 0.f) return false;  // (a sink without a value, bounded scores: the kernel that takes every form)
   return dtype == kBF16 && dv == d && op.i[5] > 0 && me_attention_mfma_supported(d, bs) && nh / nkv <= 16 && out_row % 4 == 0 &&
          op.i[11] % 4 == 0;
 }
 
 int groups_of(int64_t v) { return v > 1 ? (int)v : 1; }
+bool act_code_is_ungated(int code) { return code >= 16; }  // csrc/common.h: MeAct
 float scale_of(float f) { return f == 0.f ? 1.f : f; }
 
 class Run {
@@ -308,6 +310,21 @@ class Run {
       case kOpRoutedFF:
         routed_ff(op);
         break;
+      case kOpResultNorm:
+        result_norm(op);
+        break;
+      case kOpTokenGate: {
+        const bool fed = s_.fed && fed_tokens_;
+        ok(me_token_gate(bufs_[op.in], op.p[0], idx(s_.lay.token_ids), fed ? idx(s_.lay.token_source) : nullptr, fed ? fed_tokens_ : nullptr,
+                         bufs_[op.out], t_, (int)values_[op.in].cols, op.i[1], (int)op.i[0], prog_.vocab(), (int)op.i[2], dtype_, stream_));
+        break;
+      }
+      case kOpActivate:
+        ok(me_act_rows(bufs_[op.in], bufs_[op.out], (long long)t_ * values_[op.in].cols, (int)op.i[0], dtype_, stream_));
+        break;
+      case kOpTimeMix:
+        time_mix(op);
+        break;
       default:
         throw Error(kBadValue, "unknown operation in a step program");
     }
@@ -334,6 +351,35 @@ class Run {
                         dtype_, stream_));
     pending_ = Pending();
     release_parts();
+  }
+
+  // x += scale * rmsnorm(pending) * w; out = x in the compute dtype (a block that norms its sublayers' results).
+  void result_norm(const Op& op) {
+    if (held_.any() || pending_.carried()) throw Error(kBroken, "a result was set aside or added itself before the norm of a sublayer's result");
+    if (pending_.any() && !op.p[0]) throw Error(kBadValue, "a sublayer's result without a norm weight");
+    ok(me_result_norm_add(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, (const float*)op.p[0],
+                          op.out >= 0 ? bufs_[op.out] : nullptr, t_, h_, op.f[0], pending_.scale, dtype_, stream_));
+    pending_ = Pending();
+    release_parts();
+  }
+
+  // Time mixing: blends of neighbouring tokens, five products, the decay, the scan over the items' tokens, norm and gate.
+  void time_mix(const Op& op) {
+    const int heads = (int)op.i[0], d = (int)op.i[1], rank = (int)op.i[2], n = heads * d;
+    const long long state_row = op.i[4], prev_at = op.i[5];
+    void* mixes[5];
+    for (int i = 0; i < 5; ++i) mixes[i] = arena_.take((size_t)t_ * h_ * elem_);
+    void* proj[4];
+    for (int i = 0; i < 4; ++i) proj[i] = arena_.take((size_t)t_ * n * elem_);
+    void* z = arena_.take((size_t)t_ * rank * elem_);
+    void* ws = arena_.take((size_t)me_time_mix_workspace(t_, heads, d));
+    ok(me_time_shift(bufs_[op.in], (float*)op.p[7], state_row, prev_at, idx(s_.lay.state_slots), idx(s_.lay.item_start), idx(s_.lay.token_item),
+                     idx(s_.lay.positions), (const float*)op.p[0], mixes, t_, s_.lay.items, h_, dtype_, stream_));
+    for (int i = 0; i < 4; ++i) product(mixes[i], (const char*)op.p[1] + (size_t)i * n * h_ * elem_, n, h_, 0, dtype_, proj[i]);
+    product(mixes[4], op.p[2], rank, h_, 0, dtype_, z);
+    ok(me_time_mix(proj[0], proj[1], proj[2], proj[3], z, op.p[3], (const float*)op.p[4], (const float*)op.p[5], (const float*)op.p[6],
+                   (float*)op.p[7], state_row, idx(s_.lay.state_slots), idx(s_.lay.item_start), bufs_[op.out], values_[op.out].cols, (int)op.i[3],
+                   op.f[1], t_, s_.lay.items, heads, d, rank, op.f[0], dtype_, ws, stream_));
   }
 
   void release_parts() {
@@ -726,7 +772,8 @@ class Run {
       throw Error(kBadValue, "the rotary table covers " + std::to_string(op.i[7]) + " positions, the step may reach " +
                                  std::to_string(s_.max_ctx));
     // (the rows may be padded behind the gates, so that every row starts at a multiple of 16 bytes)
-    const long long used = (long long)nh * (d + r) + dk + nh, row = values_[op.in].cols;
+    const bool reads_only = op.i[9] != 0;  // another layer's pages: the rows hold no latent projection
+    const long long used = (long long)nh * (d + r) + (reads_only ? 0 : dk) + nh, row = values_[op.in].cols;
     if (row < used) throw Error(kBadValue, "the projections of a latent attention layer have the wrong width");
     const int32_t* table = idx(s_.lay.tables[g]);
     const int width = s_.lay.widths[g], items = s_.lay.items;
@@ -737,8 +784,8 @@ class Run {
     void* qa = arena_.take((size_t)t_ * nh * dk * elem_);
     void* ol = arena_.take((size_t)t_ * nh * vr * elem_);
     const void *kc = op.p[2], *vc = op.p[3];
-    ok(me_latent_prepare(proj, row, (const float*)op.p[0], (const float*)op.p[1], idx(s_.lay.positions), idx(s_.lay.token_item), table,
-                         width, qa, (void*)kc, (void*)vc, t_, nh, d, r, rank, vr, bs, op.f[0], dtype_, stream_));
+    ok(me_latent_prepare_for(proj, row, (const float*)op.p[0], (const float*)op.p[1], idx(s_.lay.positions), idx(s_.lay.token_item), table,
+                             width, qa, (void*)kc, (void*)vc, t_, nh, d, r, rank, vr, bs, op.f[0], reads_only ? 0 : 1, dtype_, stream_));
     ok(me_head_product(proj, row, d + r, op.p[4], qa, (long long)nh * dk, dk, nullptr, 0, t_, nh, rank, d, dtype_, stream_));
     if (latent_takes_matrix_cores(op, dtype_) && s_.decode_only) {
       // one new token per item: the split-context kernel; all heads share the one key/value head, 16 to a wave
@@ -788,11 +835,17 @@ class Run {
     float* parts = (float*)arena_.take((size_t)sums * t_ * h_ * 4);
     released_to_ = arena_.used;  // the partial sums outlive this operation, its workspace does not
     void* ws = arena_.take((size_t)me_routed_ff_workspace(t_, E, top, ff, elem_));
-    float* shared_gate = shared_ff > 0 ? (float*)arena_.take((size_t)t_ * 4) : nullptr;
-    ok(me_routed_ff_scored(bufs_[op.in], (const float*)op.p[0], op.p[1], op.p[2], parts, ws, t_, h_, E, top, ff, (int)op.i[3], op.f[0],
+    float* shared_gate = shared_ff > 0 && !op.i[9] ? (float*)arena_.take((size_t)t_ * 4) : nullptr;
+    ok(me_routed_ff_routed(bufs_[op.in], (const float*)op.p[0], op.p[1], op.p[2], parts, ws, t_, h_, E, top, ff, (int)op.i[3], op.f[0],
                            (int)op.i[4], (int)std::max<int64_t>(op.i[5], 1), (int)std::max<int64_t>(op.i[6], 1), scale_of(op.f[1]),
-                           shared_gate, dtype_, stream_));
-    if (shared_ff > 0) {
+                           shared_gate, (int)op.i[8], (const float*)op.p[5], dtype_, stream_));
+    if (shared_ff > 0 && act_code_is_ungated((int)op.i[3])) {  // an expert without a gate: up, the activation, down
+      void* up = arena_.take((size_t)t_ * shared_ff * elem_);
+      product(bufs_[op.in], op.p[3], shared_ff, h_, 0, dtype_, up);
+      if (shared_gate) throw Error(kBadValue, "a shared expert without gate rows has no gate of its own either");
+      ok(me_act_rows(up, up, (long long)t_ * shared_ff, (int)op.i[3], dtype_, stream_));
+      product(up, op.p[4], h_, shared_ff, 0, kF32, parts + (size_t)top * t_ * h_);
+    } else if (shared_ff > 0) {
       void* gu = arena_.take((size_t)t_ * 2 * shared_ff * elem_);
       void* act = arena_.take((size_t)t_ * shared_ff * elem_);
       product(bufs_[op.in], op.p[3], 2 * shared_ff, h_, 0, dtype_, gu);
@@ -814,6 +867,18 @@ class Run {
     const int width = s_.lay.widths[g];
     const long long row = values_[op.in].cols, out_row = values_[op.out].cols;
     void* q = arena_.take((size_t)t_ * nh * d * elem_);
+    const int rotary = (int)op.i[12], taps = (int)op.i[14];
+    const float* sink = (const float*)op.p[9];
+    const float softcap = op.f[3];
+    if (rotary > 0 && op.i[13] < s_.max_ctx)
+      throw Error(kBadValue, "the rotary table covers " + std::to_string(op.i[13]) + " positions, the step may reach " + std::to_string(s_.max_ctx));
+    if (rotary > 0 || taps > 0) {
+      if (pool > 0 || op.i[10] < 0) throw Error(kBadValue, "a convolution or a rotation ahead of attention with pooled blocks or without a value projection");
+      ok(me_conv_norm_rope_scatter(bufs_[op.in], row, (int)op.i[8], (int)op.i[9], (int)op.i[10], (const float*)op.p[7], taps, (float*)op.p[8],
+                                   idx(s_.lay.state_slots), idx(s_.lay.item_start), (const float*)op.p[0], (const float*)op.p[1],
+                                   (const float*)op.p[6], rotary, idx(s_.lay.positions), idx(s_.lay.token_item), table, width, q, (void*)op.p[2],
+                                   (void*)op.p[3], t_, s_.lay.items, nh, nkv, d, dv, bs, op.f[0], dtype_, stream_));
+    } else
     ok(me_whole_norm_scatter_step(bufs_[op.in], row, (int)op.i[8], (int)op.i[9], (int)op.i[10], (const float*)op.p[0],
                                   (const float*)op.p[1], idx(s_.lay.positions), idx(s_.lay.token_item), table, width, q, (void*)op.p[2],
                                   (void*)op.p[3], (void*)op.p[4], (void*)op.p[5], t_, nh, nkv, d, dv, bs, pool, op.f[0],
@@ -848,9 +913,9 @@ class Run {
                                           op.f[1], p.columns, stream_));
       return;
     }
-    ok(me_attention_general_pooled(q, op.p[2], op.p[3], idx(s_.lay.positions), idx(s_.lay.token_item), table, width, bufs_[op.out], t_, nh,
-                                   nkv, d, dv, bs, window, 0, nullptr, 0, op.f[1], nullptr, nullptr, 0, op.p[4], op.p[5], pool, out_row,
-                                   (int)op.i[11], out_scale, dtype_, s_.lay.items, stream_));
+    ok(me_attention_general_capped(q, op.p[2], op.p[3], idx(s_.lay.positions), idx(s_.lay.token_item), table, width, bufs_[op.out], t_, nh,
+                                   nkv, d, dv, bs, window, 0, nullptr, 0, op.f[1], sink, nullptr, 0, op.p[4], op.p[5], pool, out_row,
+                                   (int)op.i[11], out_scale, softcap, dtype_, s_.lay.items, stream_));
   }
 
   // Linear attention by the generalized delta rule over the state rows of the step's items (csrc/delta_rule.hip).
@@ -1022,6 +1087,9 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
     if (op.kind == kOpRoutedFF)
       need = (size_t)(op.i[1] + 1) * tokens * hidden_ * 4 + (size_t)me_routed_ff_workspace(tokens, (int)op.i[0], (int)op.i[1], (int)op.i[2], (int)elem) +
              (size_t)tokens * (4 + 3 * op.i[7] * elem + 2 * op.i[7] * 4) + 6 * pad;
+    if (op.kind == kOpTimeMix)
+      need = (size_t)tokens * (5 * hidden_ + 4 * op.i[0] * op.i[1] + op.i[2]) * elem + (size_t)me_time_mix_workspace(tokens, (int)op.i[0], (int)op.i[1]) +
+             12 * pad;
     if (op.kind == kOpDeltaRule && tokens > items) need = (size_t)me_delta_rule_workspace(tokens, (int)op.i[0], (int)op.i[1]) + pad;
     if (op.kind == kOpPooledAttention) {
       need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;

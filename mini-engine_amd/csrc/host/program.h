@@ -83,12 +83,32 @@ enum OpKind {
                       // (heads * d each), i8 the decay's inner projection (i2 wide); p0 the decay's outer weight [heads * d, i2], p1 its
                       // bias, p2 the bias of a, p3 weight of the output norm (float32 [heads * d] each), p4 state rows [slots, heads, d, d];
                       // i0 heads, i1 d; f0 eps, f1 the decay's coefficient, f2 what multiplies the result -> out, at column i9
+  kOpResultNorm = 22, // a block that norms a sublayer's result, not its input: x += scale * rmsnorm(pending) * p0 (f0 eps; the scale is the
+                      // pending result's), then out (or -1) = x in the compute dtype, which the next sublayer reads. Nothing pending
+                      // (p0 may be null): only x -> out
+  kOpTokenGate = 23,  // in z [tokens, n]; p0 a table [vocab, i1] in the compute dtype; out [tokens, n] = act(z) * table[token, i0 .. i0 + n - 1],
+                      // i2 the activation's code (MeAct)
+  kOpActivate = 24,   // in -> out (the same value or another of its size): act(in) elementwise, i0 the activation's code (MeAct)
+  kOpTimeMix = 25,    // linear attention with a decay per token and channel and a bonus for the current token (csrc/time_mix.hip). in: the
+                      // sublayer's input [tokens, hidden]; p0 float32 [5, hidden] the blends' mu (r, k, v, gate, decay), p1 W [4 n, hidden] (the rows
+                      // of r, k, v, gate), p2 W1 [i2, hidden], p3 W2 [n, i2], p4 w0, p5 bonus, p6 weight of the output norm (float32 [n]
+                      // each), p7 state rows float32 [slots, i4]: S [heads, d, d], then at i5 the input of the sequence's last token;
+                      // i0 heads, i1 d (n = i0 * i1), i2 the decay's inner size, i3 the result's column in out; f0 eps, f1 what multiplies the result
 };
+// kOpPooledAttention beyond i11: p6 a rotary table [positions, 2, i12 / 2] (i13 positions) that q and k are turned by behind their norm
+// (pairs of halves), i12 the turned elements of a head; i14 taps of a short causal convolution over time on every channel of q, k and
+// v ahead of the norm, p7 its weights float32 [nq + nk + nv, taps], p8 its state rows float32 [slots, (taps - 1) (nq + nk + nv)];
+// p9 float32 [heads] logits that count once in the softmax's denominator and have no value (null: none); f3 > 0: scores are bounded,
+// f3 * tanh(score / f3).
+// kOpLatentAttention i9 != 0: the layer reads another layer's pages; its rows hold no latent projection ([heads (d + r) | heads]).
+// kOpRoutedFF i8: identity experts (router outputs behind the experts' that stand for the token's input itself), p5 float32 correction
+// added to the scores for the choice alone (scoring 2: softmax over all outputs); i9 != 0: the shared expert has no gate of its own.
+// An activation code of MeAct (16 and more): the experts have no gate rows, p1 is [E, ff, hidden], p3 [i7, hidden].
 // kOpLinearDelta i2: the result stays pending whatever the step's size (no product adds itself to the stream).
 // kOpAttention beyond i12: i13 every (0: none) and f2 coef of a temperature on the queries, 1 + coef * ln(floor((position + 1) / every)
 // + 1); i14: the input ends in one more column per head, a gate whose sigmoid multiplies the head's output.
 
-constexpr int kOpPtrs = 8;
+constexpr int kOpPtrs = 12;
 
 constexpr int kOpInts = 16, kOpFloats = 4;
 
@@ -107,7 +127,7 @@ typedef int (*CallFn)(const CallFrame*);
 
 struct Op {
   int kind = 0, in = -1, out = -1;
-  const void* p[kOpPtrs] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+  const void* p[kOpPtrs] = {nullptr};
   int64_t i[kOpInts] = {0};
   float f[kOpFloats] = {0.f, 0.f, 0.f, 0.f};
 };

@@ -199,4 +199,34 @@ int me_delta_rule_steps(const void* proj, long long row, int c_r, int c_k, int c
 int me_sample_chunks(int vocab);
 int me_sample(const float* logits, int num_rows, int vocab, const float* temperatures, const uint64_t* keys, int* out,
               void* workspace, hipStream_t stream);
+int me_attention_general_capped(const void* q, const void* k_cache, const void* v_cache, const int* positions, const int* token_item,
+                                const int* block_table, int table_width, void* out, int num_tokens, int nh, int nkv, int d, int dv,
+                                int bs, int window, int keep_first, const float* unturn, int un_pairing, float scale, const float* sink,
+                                const void* gate, long long gate_row, const void* k_pool, const void* v_pool, int pool,
+                                long long out_row, int out_col, float out_scale, float softcap, int dtype, int items, hipStream_t stream);
+int me_latent_prepare_for(const void* proj, long long row_stride, const float* norm_w, const float* rope, const int* positions,
+                          const int* token_item, const int* block_table, int table_width, void* qa, void* k_cache, void* v_cache,
+                          int num_tokens, int nh, int d, int r, int rank, int v_rows, int bs, float eps, int writes, int dtype,
+                          hipStream_t stream);
+int me_routed_ff_routed(const void* h, const float* Wr, const void* W_gu, const void* W_down, float* parts, void* workspace, int num_tokens,
+                        int hidden, int E, int top, int ff, int act, float limit, int scoring, int n_groups, int keep_groups,
+                        float route_scale, float* shared_gate, int n_identity, const float* correction, int dtype, hipStream_t stream);
+int me_result_norm_add(float* x, const void* delta, const float* parts, int num_parts, long long part_stride, const float* w, void* h,
+                       int num_tokens, int dim, float eps, float scale, int dtype, hipStream_t stream);
+int me_token_gate(const void* z, const void* table, const int* ids, const int* fed_rows, const int* fed_tokens, void* out, int num_tokens,
+                  int n, long long table_row, int col0, int vocab, int act, int dtype, hipStream_t stream);
+int me_act_rows(const void* in, void* out, long long total, int act, int dtype, hipStream_t stream);
+int me_conv_norm_rope_scatter(const void* proj, long long row, int c_q, int c_k, int c_v, const float* conv_w, int taps, float* state,
+                              const int* state_slots, const int* item_start, const float* q_w, const float* k_w, const float* rope,
+                              int rotary, const int* positions, const int* token_item, const int* block_table, int table_width,
+                              void* q_out, void* k_cache, void* v_cache, int num_tokens, int items, int nh, int nkv, int d, int dv, int bs,
+                              float eps, int dtype, hipStream_t stream);
+int me_time_shift(const void* h, float* state, long long state_row, long long prev_at, const int* state_slots, const int* item_start,
+                  const int* token_item, const int* positions, const float* mu, void* const* outs, int num_tokens, int items, int width,
+                  int dtype, hipStream_t stream);
+long long me_time_mix_workspace(long long tokens, int heads, int d);
+int me_time_mix(const void* r, const void* k, const void* v, const void* gate, const void* z, const void* W2, const float* w0,
+                const float* bonus, const float* norm_w, float* state, long long state_row, const int* state_slots, const int* item_start,
+                void* out, long long out_row, int out_col, float out_scale, int num_tokens, int items, int heads, int d, int rank, float eps,
+                int dtype, void* workspace, hipStream_t stream);
 }

@@ -21,19 +21,20 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
     const T* __restrict__ proj, size_t row_stride, const float* __restrict__ norm_w, const float* __restrict__ rope,
     const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table, int table_width,
     T* __restrict__ qa, T* __restrict__ k_cache, T* __restrict__ v_cache, int nh, int d, int r, int rank, int v_rows, int bs,
-    float eps) {
+    float eps, int writes) {
   __shared__ float scratch[16];
   const int t = blockIdx.x, dk = rank + r, half = r / 2;
   const int pos = positions[t];
-  const int page = block_table[(size_t)token_item[t] * table_width + pos / bs], slot = pos % bs;
+  const int page = writes ? block_table[(size_t)token_item[t] * table_width + pos / bs] : -1, slot = pos % bs;
   const T* row = proj + (size_t)t * row_stride;
   const T* lat = row + (size_t)nh * (d + r);
   float ss = 0.f;
-  for (int i = threadIdx.x; i < rank; i += blockDim.x) {
-    const float v = to_float(lat[i]);
-    ss = fmaf(v, v, ss);
-  }
-  const float inv = rsqrtf(block_sum(ss, scratch) / (float)rank + eps);
+  if (writes)  // (a layer that reads another layer's pages has no latent projection: its rows hold the queries alone)
+    for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+      const float v = to_float(lat[i]);
+      ss = fmaf(v, v, ss);
+    }
+  const float inv = writes ? rsqrtf(block_sum(ss, scratch) / (float)rank + eps) : 0.f;
   const float* cs = rope + (size_t)pos * r;
   if (page >= 0) {
     T* krow = k_cache + ((size_t)page * bs + slot) * dk;
@@ -62,23 +63,38 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
   }
 }
 
+// writes == 0: the layer reads another layer's pages; its rows hold no latent projection (queries, then whatever follows), nothing
+// is normed and no page is written, only the queries' turned parts.
+extern "C" int me_latent_prepare_for(const void* proj, long long row_stride, const float* norm_w, const float* rope,
+                                     const int* positions, const int* token_item, const int* block_table, int table_width, void* qa,
+                                     void* k_cache, void* v_cache, int num_tokens, int nh, int d, int r, int rank, int v_rows, int bs,
+                                     float eps, int writes, int dtype, hipStream_t stream);
+
 extern "C" int me_latent_prepare(const void* proj, long long row_stride, const float* norm_w, const float* rope,
                                  const int* positions, const int* token_item, const int* block_table, int table_width, void* qa,
                                  void* k_cache, void* v_cache, int num_tokens, int nh, int d, int r, int rank, int v_rows, int bs,
                                  float eps, int dtype, hipStream_t stream) {
+  return me_latent_prepare_for(proj, row_stride, norm_w, rope, positions, token_item, block_table, table_width, qa, k_cache, v_cache,
+                               num_tokens, nh, d, r, rank, v_rows, bs, eps, 1, dtype, stream);
+}
+
+extern "C" int me_latent_prepare_for(const void* proj, long long row_stride, const float* norm_w, const float* rope,
+                                     const int* positions, const int* token_item, const int* block_table, int table_width, void* qa,
+                                     void* k_cache, void* v_cache, int num_tokens, int nh, int d, int r, int rank, int v_rows, int bs,
+                                     float eps, int writes, int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (nh <= 0 || d <= 0 || rank <= 0 || r <= 0 || r % 2) return me_fail("me_latent_prepare: heads=%d d=%d rank=%d rot=%d", nh, d, rank, r);
   if (v_rows != rank && v_rows != rank + r) return me_fail("me_latent_prepare: value pages of %d rows for a latent of %d + %d", v_rows, rank, r);
-  if (row_stride < (long long)nh * (d + r) + rank + r) return me_fail("me_latent_prepare: rows of %lld elements are too short", row_stride);
+  if (row_stride < (long long)nh * (d + r) + (writes ? rank + r : 0)) return me_fail("me_latent_prepare: rows of %lld elements are too short", row_stride);
   if (bs <= 0 || table_width <= 0) return me_fail("me_latent_prepare: block_size=%d table_width=%d", bs, table_width);
   if (dtype == ME_F32)
     latent_prepare_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)proj, (size_t)row_stride, norm_w, rope, positions,
                                                                  token_item, block_table, table_width, (float*)qa, (float*)k_cache,
-                                                                 (float*)v_cache, nh, d, r, rank, v_rows, bs, eps);
+                                                                 (float*)v_cache, nh, d, r, rank, v_rows, bs, eps, writes);
   else
     latent_prepare_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)proj, (size_t)row_stride, norm_w, rope, positions,
                                                                   token_item, block_table, table_width, (bf16_t*)qa,
-                                                                  (bf16_t*)k_cache, (bf16_t*)v_cache, nh, d, r, rank, v_rows, bs, eps);
+                                                                  (bf16_t*)k_cache, (bf16_t*)v_cache, nh, d, r, rank, v_rows, bs, eps, writes);
   return me_check_launch("me_latent_prepare");
 }
 

@@ -1,0 +1,206 @@
+// Linear attention with a decay per token, head and key channel and a bonus for the current token (the time mixing of RWKV-6),
+// a d x d float32 state per request and head:
+//
+//     o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t,        S_t = diag(w_t) S_(t-1) + k_t v_t^T
+//
+// Every projection reads a blend of the token's input and the input of the token before it, h + (h' - h) * mu, with a mu of its own.
+//
+//   shift    for every token the five blends (r, k, v, gate, decay) in the activations' type; h' of an item's first token is the
+//            item's state row (zeros at position 0). A second launch keeps the item's last input as the next h'.
+//   decay    w = exp(-exp(W_2 tanh(z) + w_0)) in float32 for all tokens, z the decay's inner projection.
+//   scan     a wave per (item, head, 16 value channels): lane (p, c) holds a quarter of the rows of column c of S and walks the
+//            item's tokens; the quarters' sums meet through two exchanges. Sums run in an order that the head's size alone
+//            fixes, so a token's result does not depend on how the sequence was cut or on what else the step holds.
+//   finish   every head's o over its root mean square, times a weight, times silu(gate), times the caller's scale.
+//
+// State row of a slot: [heads, d (key), d (value)] float32, then the `width` elements of h'.
+#include "common.h"
+
+template <typename T>
+__global__ __launch_bounds__(256) void time_shift_kernel(const T* __restrict__ h, const float* __restrict__ state, long long state_row,
+                                                         long long prev_at, const int* __restrict__ state_slots,
+                                                         const int* __restrict__ item_start, const int* __restrict__ token_item,
+                                                         const int* __restrict__ positions, const float* __restrict__ mu,
+                                                         T* __restrict__ o0, T* __restrict__ o1, T* __restrict__ o2, T* __restrict__ o3,
+                                                         T* __restrict__ o4, int width) {
+  const int t = blockIdx.x, item = token_item[t];
+  const bool from_state = t == item_start[item];
+  const float* prev_row = state + (size_t)state_slots[item] * state_row + prev_at;
+  const bool none = positions[t] == 0;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float x = to_float(h[(size_t)t * width + i]);
+    const float prev = none ? 0.f : (from_state ? prev_row[i] : to_float(h[(size_t)(t - 1) * width + i]));
+    const float dlt = prev - x;
+    const size_t at = (size_t)t * width + i;
+    o0[at] = from_float<T>(fmaf(dlt, mu[i], x));
+    o1[at] = from_float<T>(fmaf(dlt, mu[width + i], x));
+    o2[at] = from_float<T>(fmaf(dlt, mu[2 * width + i], x));
+    o3[at] = from_float<T>(fmaf(dlt, mu[3 * width + i], x));
+    o4[at] = from_float<T>(fmaf(dlt, mu[4 * width + i], x));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void time_shift_keep_kernel(const T* __restrict__ h, float* __restrict__ state, long long state_row,
+                                                              long long prev_at, const int* __restrict__ state_slots,
+                                                              const int* __restrict__ item_start, int width) {
+  const int item = blockIdx.x, last = item_start[item + 1] - 1;
+  if (last < item_start[item]) return;
+  float* prev_row = state + (size_t)state_slots[item] * state_row + prev_at;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) prev_row[i] = to_float(h[(size_t)last * width + i]);
+}
+
+// h [T, width]; mu float32 [5, width] (r, k, v, gate, decay); outs: five [T, width] buffers in the activations' type.
+extern "C" int me_time_shift(const void* h, float* state, long long state_row, long long prev_at, const int* state_slots,
+                             const int* item_start, const int* token_item, const int* positions, const float* mu, void* const* outs,
+                             int num_tokens, int items, int width, int dtype, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (width <= 0 || prev_at < 0 || prev_at + width > state_row) return me_fail("me_time_shift: width=%d at %lld of a row of %lld", width, prev_at, state_row);
+  if (dtype == ME_F32) {
+    time_shift_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)h, state, state_row, prev_at, state_slots, item_start, token_item,
+                                                             positions, mu, (float*)outs[0], (float*)outs[1], (float*)outs[2],
+                                                             (float*)outs[3], (float*)outs[4], width);
+    time_shift_keep_kernel<float><<<items, 256, 0, stream>>>((const float*)h, state, state_row, prev_at, state_slots, item_start, width);
+  } else {
+    time_shift_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)h, state, state_row, prev_at, state_slots, item_start,
+                                                              token_item, positions, mu, (bf16_t*)outs[0], (bf16_t*)outs[1],
+                                                              (bf16_t*)outs[2], (bf16_t*)outs[3], (bf16_t*)outs[4], width);
+    time_shift_keep_kernel<bf16_t><<<items, 256, 0, stream>>>((const bf16_t*)h, state, state_row, prev_at, state_slots, item_start, width);
+  }
+  return me_check_launch("me_time_shift");
+}
+
+// decay[t, c] = exp(-exp(sum_j W2[c, j] tanh(z[t, j]) + w0[c])). Grid (tokens), a thread a channel in turns.
+#define TM_MAX_RANK 256
+template <typename T>
+__global__ __launch_bounds__(256) void time_decay_kernel(const T* __restrict__ z, const T* __restrict__ W2, const float* __restrict__ w0,
+                                                         float* __restrict__ decay, int n, int rank) {
+  __shared__ float th[TM_MAX_RANK];
+  const int t = blockIdx.x;
+  for (int j = threadIdx.x; j < rank; j += blockDim.x) th[j] = tanhf(to_float(z[(size_t)t * rank + j]));
+  __syncthreads();
+  for (int c = threadIdx.x; c < n; c += blockDim.x) {
+    const T* wr = W2 + (size_t)c * rank;
+    float s = 0.f;
+    for (int j = 0; j < rank; ++j) s = fmaf(to_float(wr[j]), th[j], s);
+    decay[(size_t)t * n + c] = expf(-expf(s + w0[c]));
+  }
+}
+
+// A wave per (item, head, group of 16 value channels); RPL: rows of S a lane holds (d <= 4 * RPL).
+template <typename T, int RPL>
+__global__ __launch_bounds__(64) void time_scan_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v,
+                                                       const float* __restrict__ decay, const float* __restrict__ bonus,
+                                                       float* __restrict__ state, long long state_row, const int* __restrict__ state_slots,
+                                                       const int* __restrict__ item_start, float* __restrict__ o, int heads, int d) {
+  const int groups = (d + 15) / 16;
+  const int item = blockIdx.x / (heads * groups), head = (blockIdx.x / groups) % heads, grp = blockIdx.x % groups;
+  const int lane = threadIdx.x, p = lane >> 4, c = grp * 16 + (lane & 15);
+  const int per = (d + 3) / 4, i0 = p * per;
+  const int first = item_start[item], end = item_start[item + 1];
+  const bool col = c < d;
+  const int n = heads * d;
+  float* S = state + (size_t)state_slots[item] * state_row + (size_t)head * d * d;
+  float s[RPL], u[RPL];
+#pragma unroll
+  for (int a = 0; a < RPL; ++a) {
+    const int i = i0 + a;
+    const bool there = a < per && i < d;
+    s[a] = there && col ? S[(size_t)i * d + c] : 0.f;
+    u[a] = there ? bonus[head * d + i] : 0.f;
+  }
+  for (int t = first; t < end; ++t) {
+    const size_t at = (size_t)t * n + head * d;
+    const float vc = col ? to_float(v[at + c]) : 0.f;
+    float rr[RPL], kk[RPL], ww[RPL];
+#pragma unroll
+    for (int a = 0; a < RPL; ++a) {
+      const int i = i0 + a;
+      const bool there = a < per && i < d;
+      rr[a] = there ? to_float(r[at + i]) : 0.f;
+      kk[a] = there ? to_float(k[at + i]) : 0.f;
+      ww[a] = there ? decay[at + i] : 0.f;
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int a = 0; a < RPL; ++a) {
+      const float kv = kk[a] * vc;
+      acc = fmaf(rr[a], fmaf(u[a], kv, s[a]), acc);
+      s[a] = fmaf(ww[a], s[a], kv);
+    }
+    acc += __shfl_xor(acc, 16, ME_WAVE);
+    acc += __shfl_xor(acc, 32, ME_WAVE);
+    if (p == 0 && col) o[at + c] = acc;
+  }
+#pragma unroll
+  for (int a = 0; a < RPL; ++a) {
+    const int i = i0 + a;
+    if (a < per && i < d && col) S[(size_t)i * d + c] = s[a];
+  }
+}
+
+// A wave per (token, head): o over its root mean square, times the weight, silu(gate) and the scale, into out at column out_col.
+template <typename T>
+__global__ __launch_bounds__(256) void time_finish_kernel(const float* __restrict__ o, const T* __restrict__ gate, const float* __restrict__ w,
+                                                          T* __restrict__ out, long long out_row, int out_col, float out_scale,
+                                                          long long units, int heads, int d, float eps) {
+  const long long unit = (long long)blockIdx.x * (blockDim.x / ME_WAVE) + threadIdx.x / ME_WAVE;
+  if (unit >= units) return;
+  const int lane = threadIdx.x & (ME_WAVE - 1);
+  const long long t = unit / heads;
+  const int head = (int)(unit % heads), n = heads * d;
+  const float* orow = o + (size_t)t * n + head * d;
+  float ss = 0.f;
+  for (int i = lane; i < d; i += ME_WAVE) ss = fmaf(orow[i], orow[i], ss);
+  const float rinv = rsqrtf(wave_sum(ss) / (float)d + eps) * out_scale;
+  for (int i = lane; i < d; i += ME_WAVE) {
+    const float g = to_float(gate[(size_t)t * n + head * d + i]);
+    out[(size_t)t * out_row + out_col + head * d + i] = from_float<T>(orow[i] * rinv * w[head * d + i] * (g / (1.f + expf(-g))));
+  }
+}
+
+extern "C" long long me_time_mix_workspace(long long tokens, int heads, int d) { return 2 * tokens * heads * d * 4 + 512; }
+
+// r, k, v, gate [T, heads * d] and z [T, rank] in the activations' type; W2 [heads * d, rank] in the activations' type; w0, bonus,
+// norm_w float32 [heads * d]; state float32 rows of state_row elements whose first heads * d * d are S. out [T, out_row], the
+// result at column out_col. workspace: me_time_mix_workspace bytes.
+extern "C" int me_time_mix(const void* r, const void* k, const void* v, const void* gate, const void* z, const void* W2, const float* w0,
+                           const float* bonus, const float* norm_w, float* state, long long state_row, const int* state_slots,
+                           const int* item_start, void* out, long long out_row, int out_col, float out_scale, int num_tokens, int items,
+                           int heads, int d, int rank, float eps, int dtype, void* workspace, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads <= 0 || d <= 0 || d > 256) return me_fail("me_time_mix: %d heads of %d elements (at most 256)", heads, d);
+  if (rank <= 0 || rank > TM_MAX_RANK) return me_fail("me_time_mix: a decay of inner size %d (at most %d)", rank, TM_MAX_RANK);
+  const long long n = (long long)heads * d;
+  if (out_col < 0 || out_col + n > out_row) return me_fail("me_time_mix: the result at column %d of a row of %lld", out_col, out_row);
+  if ((long long)heads * d * d > state_row) return me_fail("me_time_mix: state rows of %lld elements", state_row);
+  float* decay = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  float* o = decay + (size_t)num_tokens * n;
+  const unsigned scan_blocks = (unsigned)(items * heads * ((d + 15) / 16));
+  const long long units = (long long)num_tokens * heads;
+  const unsigned fin_blocks = (unsigned)((units + 3) / 4);
+#define ME_TM_RUN(TT)                                                                                                               \
+  do {                                                                                                                              \
+    time_decay_kernel<TT><<<num_tokens, 256, 0, stream>>>((const TT*)z, (const TT*)W2, w0, decay, (int)n, rank);                    \
+    if (d <= 32)                                                                                                                    \
+      time_scan_kernel<TT, 8><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
+                                                              state_slots, item_start, o, heads, d);                                \
+    else if (d <= 64)                                                                                                               \
+      time_scan_kernel<TT, 16><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
+                                                               state_slots, item_start, o, heads, d);                               \
+    else if (d <= 128)                                                                                                              \
+      time_scan_kernel<TT, 32><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
+                                                               state_slots, item_start, o, heads, d);                               \
+    else                                                                                                                            \
+      time_scan_kernel<TT, 64><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
+                                                               state_slots, item_start, o, heads, d);                               \
+    time_finish_kernel<TT><<<fin_blocks, 256, 0, stream>>>(o, (const TT*)gate, norm_w, (TT*)out, out_row, out_col, out_scale, units,  \
+                                                           heads, d, eps);                                                          \
+  } while (0)
+  if (dtype == ME_F32)
+    ME_TM_RUN(float);
+  else
+    ME_TM_RUN(bf16_t);
+#undef ME_TM_RUN
+  return me_check_launch("me_time_mix");
+}

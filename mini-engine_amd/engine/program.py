@@ -29,9 +29,10 @@ _vp, _i64, _i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 _declared = False
 
 (EMBED, NORM_LINEAR, NORM, LINEAR, LINEAR_DELTA, DELTA, ATTENTION, HEAD, SAMPLE, ADD, CALL, HEAD_ROWS, DECAY_STATE, HOLD, STREAMS,
- STREAM_NORM, STREAM_HEAD, LATENT_ATTENTION, ROUTED_FF, STREAM_NORM_LINEAR, POOLED_ATTENTION, DELTA_RULE) = range(22)
-ROUTER_SCORINGS = {"softmax_picked": 0, "sigmoid_normalized": 1}  # csrc/routed_ff.hip: RF_SCORE_*
-OP_PTRS, OP_INTS, OP_FLOATS = 8, 16, 4  # csrc/host/program.h: kOpPtrs, kOpInts, kOpFloats
+ STREAM_NORM, STREAM_HEAD, LATENT_ATTENTION, ROUTED_FF, STREAM_NORM_LINEAR, POOLED_ATTENTION, DELTA_RULE, RESULT_NORM, TOKEN_GATE,
+ ACTIVATE, TIME_MIX) = range(26)
+ROUTER_SCORINGS = {"softmax_picked": 0, "sigmoid_normalized": 1, "softmax_all": 2}  # csrc/routed_ff.hip: RF_SCORE_*
+OP_PTRS, OP_INTS, OP_FLOATS = 12, 16, 4  # csrc/host/program.h: kOpPtrs, kOpInts, kOpFloats
 MAX_STREAMS = 8  # csrc/streams.hip: ME_MAX_STREAMS
 _RAISES = {1: ValueError, 2: RuntimeError, 3: AssertionError}
 
@@ -193,6 +194,9 @@ class StepProgram:
         self.num_streams = 0  # residual streams of a token (0: the one plain stream)
         self._stream_rewrite: torch.Tensor | None = None  # how the pending result rewrites the streams (mix, then out)
         self.draws = False
+        # the residual stream in the compute dtype as the last norm of a sublayer's result left it (a value that no scope owns), for
+        # blocks whose sublayers read the stream itself
+        self.stream_value: int | None = None
         self.last_prefill_columns = 0  # query columns of the prefill attention's blocks in the last eager step (0: none ran)
         # called parts: their C trampolines (kept alive), the memory and the batch of the step that is running,
         # and the exception a call raised (raised again once the step's call into C++ has come back)
@@ -207,9 +211,9 @@ class StepProgram:
             self._L.me_runner_delete(handle)
 
     # ------------------------------------------------------------------ values
-    def take(self, cols: int, elem: int | None = None) -> int:
+    def take(self, cols: int, elem: int | None = None, scoped: bool = True) -> int:
         """A ``[tokens, cols]`` buffer (elements of the compute dtype unless ``elem`` bytes are asked for)
-        that stays the caller's until the scope it was taken in ends."""
+        that stays the caller's until the scope it was taken in ends (``scoped`` false: until the caller hands it back)."""
         key = (int(cols), int(elem or self.elem))
         pool = self._free.setdefault(key, [])
         if pool:
@@ -217,7 +221,7 @@ class StepProgram:
         else:
             v = _ok(self._L.me_runner_value(self.handle, key[0], key[1]))
             self._value_kinds.append(key)
-        if self._scopes:
+        if self._scopes and scoped:
             self._scopes[-1].append(v)
         return v
 
@@ -359,13 +363,14 @@ class StepProgram:
     def latent_attention(self, proj: int, *, latent_norm: torch.Tensor, rope: torch.Tensor, k_cache: torch.Tensor,
                          v_cache: torch.Tensor, key_map: torch.Tensor, value_map: torch.Tensor, sink: torch.Tensor | None,
                          heads: int, head_dim: int, rotary_dim: int, rank: int, value_dim: int, block_size: int, group: int,
-                         eps: float, scale: float) -> int:
+                         eps: float, scale: float, writes: bool = True) -> int:
         """Attention over one cached latent per token for a value ``[tokens, heads (head_dim + rotary_dim) | rank + rotary_dim |
         heads]`` (queries; the latent projection and the key part that all heads share; a gate per head). ``key_map`` ``[heads,
         rank, head_dim]`` (the keys' map per head, transposed) and ``value_map`` ``[heads, value_dim, rank]`` in the compute
         dtype; ``sink`` float32 ``[heads]`` or None; pages of one key/value head with keys of ``rank + rotary_dim`` and values
         of ``rank`` elements. Returns the value ``[tokens, heads * value_dim]``, gated."""
-        cols = heads * (head_dim + rotary_dim) + rank + rotary_dim + heads
+        # (``writes`` false: the pages are another layer's; the rows hold no latent projection, ``[tokens, heads (head_dim + rotary_dim) | heads]``)
+        cols = heads * (head_dim + rotary_dim) + (rank + rotary_dim if writes else 0) + heads
         if self._value_kinds[proj][0] < cols or self._value_kinds[proj][1] != self.elem:  # (columns of padding may follow)
             raise ValueError(f"the projections have {self._value_kinds[proj][0]} columns, not {cols}")
         self._want(latent_norm, torch.float32, (rank,), "weight of the latent's norm")
@@ -382,40 +387,57 @@ class StepProgram:
             raise ValueError("a latent attention layer keeps pages of one head: keys of rank + rotary_dim, values of rank (or as many) elements")
         out = self.take(heads * value_dim)
         self.op(LATENT_ATTENTION, in_=proj, out=out, ptrs=[latent_norm, rope, k_cache, v_cache, key_map, value_map, sink],
-                ints=[heads, head_dim, rotary_dim, rank, value_dim, block_size, group, rope.shape[0], value_rows], floats=[eps, scale])
+                ints=[heads, head_dim, rotary_dim, rank, value_dim, block_size, group, rope.shape[0], value_rows, int(not writes)],
+                floats=[eps, scale])
         return out
 
     def routed_ff(self, x: int, *, router: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, top_k: int, activation: str,
                   activation_limit: float = 0.0, scoring: str = "softmax_picked", num_groups: int = 1, keep_groups: int = 1,
                   route_scale: float = 1.0, shared_gate_up: torch.Tensor | None = None, shared_down: torch.Tensor | None = None,
-                  shared_limit: float = 0.0) -> None:
+                  shared_limit: float = 0.0, identity_experts: int = 0, correction: torch.Tensor | None = None,
+                  shared_gated: bool = True) -> None:
         """A feed-forward of routed experts on the value ``x`` as the part's result. ``router`` float32 ``[experts, hidden]``;
         ``gate_up`` ``[experts, 2 ff, hidden]`` (an expert's gate rows, then its up rows) and ``down`` ``[experts, hidden, ff]``
         in the compute dtype. ``scoring``, ``num_groups``, ``keep_groups``, ``route_scale``: how the picks are bounded and weighted
         (:class:`~mini_engine_amd.config.specs.RoutedExpertsSpec`). ``shared_gate_up`` ``[2 ff_s, hidden]`` and ``shared_down``
         ``[hidden, ff_s]``: an expert that every token uses; the router then has one more row behind the experts', the token's
         product with which, through a sigmoid, multiplies that expert's result."""
-        from ..ops.kernels import gate_code
+        from ..ops.kernels import UNGATED_ACTIVATIONS, gate_code
 
+        # An activation of UNGATED_ACTIVATIONS: the experts have no gate, ``gate_up`` is ``[experts, ff, hidden]`` (up rows alone) and
+        # ``shared_gate_up`` ``[ff_s, hidden]``. ``identity_experts``: that many router outputs behind the experts' stand for identity
+        # experts (the token's input itself, times the weight); ``correction`` float32 ``[experts + identity_experts]`` is added to the
+        # scores for the choice alone (scoring "softmax_all"). ``shared_gated`` false: nothing multiplies the shared expert's result.
+        ungated = activation in UNGATED_ACTIVATIONS
         experts, two_ff, hidden = gate_up.shape
+        if ungated:
+            two_ff *= 2
         if self._value_kinds[x] != (self.hidden, self.elem) or hidden != self.hidden:
             raise ValueError("routed experts read the hidden size in the compute dtype")
         shared_ff = 0
         if shared_gate_up is not None:
-            shared_ff = shared_gate_up.shape[0] // 2
-            self._want(shared_gate_up, self.dtype, (2 * shared_ff, hidden), "the shared expert's gate and up rows")
+            shared_ff = shared_gate_up.shape[0] if ungated else shared_gate_up.shape[0] // 2
+            self._want(shared_gate_up, self.dtype, ((1 if ungated else 2) * shared_ff, hidden), "the shared expert's gate and up rows")
             self._want(shared_down, self.dtype, (hidden, shared_ff), "the shared expert's down rows")
-        self._want(router, torch.float32, (experts + (1 if shared_ff else 0), hidden), "router")
+            if ungated and shared_gated:
+                raise ValueError("a shared expert without gate rows has no gate of its own either")
+        if identity_experts < 0 or (identity_experts and scoring != "softmax_all"):
+            raise ValueError("identity experts are picked by a router that scores by softmax_all")
+        if correction is not None:
+            self._want(correction, torch.float32, (experts + identity_experts,), "the scores' correction")
+        self._want(router, torch.float32, (experts + identity_experts + (1 if shared_ff and shared_gated else 0), hidden), "router")
         self._want(gate_up, self.dtype, None, "experts' gate and up rows")
         self._want(down, self.dtype, (experts, hidden, two_ff // 2), "experts' down rows")
-        if not 1 <= top_k <= experts:
-            raise ValueError(f"{top_k} of {experts} experts a token")
+        if not 1 <= top_k <= experts + identity_experts:
+            raise ValueError(f"{top_k} of {experts + identity_experts} experts a token")
         if scoring not in ROUTER_SCORINGS:
             raise ValueError(f"a router scores by one of {sorted(ROUTER_SCORINGS)}, not {scoring!r}")
         if num_groups < 1 or experts % num_groups or not 1 <= keep_groups <= num_groups or keep_groups * (experts // num_groups) < top_k:
             raise ValueError(f"{experts} experts in {num_groups} groups of which {keep_groups} are kept, {top_k} picks")
-        self.op(ROUTED_FF, in_=x, ptrs=[router, gate_up, down, shared_gate_up, shared_down],
-                ints=[experts, top_k, two_ff // 2, gate_code(activation, limited=True), ROUTER_SCORINGS[scoring], num_groups, keep_groups, shared_ff],
+        code = UNGATED_ACTIVATIONS[activation] if ungated else gate_code(activation, limited=True)
+        self.op(ROUTED_FF, in_=x, ptrs=[router, gate_up, down, shared_gate_up, shared_down, correction],
+                ints=[experts, top_k, two_ff // 2, code, ROUTER_SCORINGS[scoring], num_groups, keep_groups, shared_ff, identity_experts,
+                      int(not shared_gated)],
                 floats=[activation_limit, route_scale, shared_limit, self.delta_scale])
         self._pending_value = None
 
@@ -433,15 +455,41 @@ class StepProgram:
     def pooled_attention(self, proj: int, out: int, *, q_col: int, k_col: int, v_col: int, out_col: int, q_norm: torch.Tensor,
                          k_norm: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, k_pool: torch.Tensor | None,
                          v_pool: torch.Tensor | None, heads: int, kv_heads: int, head_dim: int, value_dim: int, block_size: int,
-                         window: int, pooled_block: int, group: int, eps: float, scale: float, out_scale: float = 1.0) -> None:
+                         window: int, pooled_block: int, group: int, eps: float, scale: float, out_scale: float = 1.0,
+                         rope: torch.Tensor | None = None, conv: torch.Tensor | None = None, conv_state: torch.Tensor | None = None,
+                         sink: torch.Tensor | None = None, softcap: float = 0.0) -> None:
         """Causal attention without rotation whose q and k are normed over their whole projection, over a window of ``window``
         keys (0: all) and, with ``pooled_block`` P > 0, the means of the whole blocks of P keys and values before the window. The
         value ``proj`` holds the queries at column ``q_col``, the keys at ``k_col`` and the values at ``v_col`` (-1: the values are
         the keys as projected); the result (``heads * value_dim`` columns, times ``out_scale``) goes to the value ``out`` at
-        column ``out_col``."""
+        column ``out_col``.
+
+        ``rope`` float32 ``[positions, 2, r/2]``: q and k are turned by the position behind their norm (the first r elements of every
+        head, element i with i + r/2). ``conv`` float32 ``[nq + nk + nv, taps]`` with ``conv_state`` float32 ``[slots, (taps - 1) (nq + nk +
+        nv)]``: a short causal convolution over time on every channel of q, k and v ahead of the norm. ``sink`` float32 ``[heads]``:
+        logits that count once in the softmax's denominator and have no value. ``softcap`` > 0: scores become ``softcap tanh(score /
+        softcap)``."""
         row, out_row = self._value_kinds[proj][0], self._value_kinds[out][0]
         if self._value_kinds[proj][1] != self.elem or self._value_kinds[out][1] != self.elem:
             raise ValueError("attention reads and writes values of the compute dtype")
+        rotary = covers = taps = 0
+        if rope is not None:
+            self._want(rope, torch.float32, None, "rotary table")
+            rotary, covers = 2 * rope.shape[2], rope.shape[0]
+            if covers < self.max_positions or rotary > head_dim:
+                raise ValueError(f"the rotary table covers {covers} positions of {self.max_positions} and {rotary} elements of {head_dim}")
+        if conv is not None:
+            channels = heads * head_dim + kv_heads * (head_dim + value_dim)
+            taps = int(conv.shape[1])
+            self._want(conv, torch.float32, (channels, taps), "the convolutions' weights")
+            if taps > 1:
+                self._want(conv_state, torch.float32, (conv_state.shape[0], (taps - 1) * channels), "the convolutions' state rows")
+        if (rope is not None or conv is not None) and (pooled_block or v_col < 0):
+            raise ValueError("a rotation or a convolution comes with a value projection and without pooled blocks")
+        if sink is not None:
+            self._want(sink, torch.float32, (heads,), "sink")
+        if softcap < 0:
+            raise ValueError("scores are bounded by a positive number")
         for col, n in ((q_col, heads * head_dim), (k_col, kv_heads * head_dim)) + (((v_col, kv_heads * value_dim),) if v_col >= 0 else ()):
             if col < 0 or col + n > row:
                 raise ValueError(f"columns {col} .. {col + n - 1} of a value of {row}")
@@ -460,9 +508,11 @@ class StepProgram:
                 raise ValueError("pooled blocks lie before a window")
             self._want(k_pool, self.dtype, tuple(k_cache.shape), "pooled key pages")
             self._want(v_pool, self.dtype, tuple(v_cache.shape), "pooled value pages")
-        self.op(POOLED_ATTENTION, in_=proj, out=out, ptrs=[q_norm, k_norm, k_cache, v_cache, k_pool, v_pool],
-                ints=[heads, kv_heads, head_dim, value_dim, block_size, window, pooled_block, group, q_col, k_col, v_col, out_col],
-                floats=[eps, scale, out_scale])
+        self.op(POOLED_ATTENTION, in_=proj, out=out,
+                ptrs=[q_norm, k_norm, k_cache, v_cache, k_pool, v_pool, rope, conv, conv_state if taps > 1 else None, sink],
+                ints=[heads, kv_heads, head_dim, value_dim, block_size, window, pooled_block, group, q_col, k_col, v_col, out_col,
+                      rotary, covers, taps],
+                floats=[eps, scale, out_scale, softcap])
 
     def delta_rule(self, proj: int, out: int, *, cols: dict, out_col: int, decay_outer: torch.Tensor, decay_bias: torch.Tensor,
                    rate_bias: torch.Tensor, norm_weight: torch.Tensor, state: torch.Tensor, heads: int, head_dim: int,
@@ -488,6 +538,70 @@ class StepProgram:
         self.op(DELTA_RULE, in_=proj, out=out, ptrs=[decay_outer, decay_bias, rate_bias, norm_weight, state],
                 ints=[heads, head_dim, decay_rank, cols["r"], cols["k"], cols["v"], cols["g"], cols["a"], cols["w1"], out_col],
                 floats=[eps, decay_coef, out_scale])
+
+    # ----------------------------------------------------------- a block that norms its sublayers' results
+    def result_normed(self, norm=None, out: bool = True) -> int:
+        """``x += rmsnorm(pending result) * weight`` (``norm`` RMS-shaped; None where nothing is pending), then the stream in the compute
+        dtype as a value, which the next sublayer reads (-1 with ``out`` false)."""
+        weight = eps = None
+        if norm is not None:
+            fused = norm.as_fused()
+            if fused is None or getattr(norm, "groups", 1) != 1:
+                raise ValueError("a sublayer's result is normed by an RMS norm without groups")
+            weight, eps = fused
+            self._want(weight, torch.float32, (self.hidden,), "norm weight")
+        value = self.take(self.hidden, self.elem, scoped=False) if out else -1
+        self.op(RESULT_NORM, out=value, ptrs=[weight], floats=[eps or 0.0])
+        self.pending_consumed()
+        if self.stream_value is not None:  # (the sublayer that read the stream as it was is done)
+            self._give_back(self.stream_value)
+        self.stream_value = value if out else None
+        return value
+
+    def token_gate(self, z: int, table: torch.Tensor, col: int, activation: str) -> int:
+        """``act(z) * table[token, col : col + n]`` for a value ``z`` ``[tokens, n]``; ``table`` ``[vocab, row]`` in the compute dtype."""
+        from ..ops.kernels import UNGATED_ACTIVATIONS
+
+        n = self._value_kinds[z][0]
+        self._want(table, self.dtype, (self.vocab, table.shape[1]), "a table of rows per token id")
+        if col < 0 or col + n > table.shape[1] or self._value_kinds[z][1] != self.elem:
+            raise ValueError(f"columns {col} .. {col + n - 1} of a table of {table.shape[1]}")
+        out = self.take(n)
+        self.op(TOKEN_GATE, in_=z, out=out, ptrs=[table], ints=[col, table.shape[1], UNGATED_ACTIVATIONS[activation]])
+        return out
+
+    def activate(self, x: int, activation: str) -> int:
+        """``act(x)`` elementwise, in place; returns ``x``."""
+        from ..ops.kernels import UNGATED_ACTIVATIONS
+
+        if activation not in UNGATED_ACTIVATIONS:
+            raise ValueError(f"an ungated feed-forward knows the activations {sorted(UNGATED_ACTIVATIONS)}, got {activation!r}")
+        self.op(ACTIVATE, in_=x, out=x, ints=[UNGATED_ACTIVATIONS[activation]])
+        return x
+
+    def time_mix(self, h: int, out: int, *, out_col: int, mu: torch.Tensor, w_rkvg: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+                 w0: torch.Tensor, bonus: torch.Tensor, norm_weight: torch.Tensor, state: torch.Tensor, heads: int, head_dim: int,
+                 eps: float, out_scale: float = 1.0) -> None:
+        """Linear attention with a decay per token and channel and a bonus for the current token, on the value ``h`` ``[tokens, hidden]``
+        (the sublayer's input). ``mu`` float32 ``[5, hidden]`` (the blends of r, k, v, gate, decay with the token before); ``w_rkvg`` ``[4 n,
+        hidden]``, ``w1`` ``[rank, hidden]``, ``w2`` ``[n, rank]`` in the compute dtype (n = heads * head_dim); ``w0``, ``bonus``, ``norm_weight``
+        float32 ``[n]``; ``state`` float32 ``[slots, heads * head_dim^2 + hidden]``. The result (times ``out_scale``) goes to ``out`` at
+        ``out_col``."""
+        n, rank = heads * head_dim, int(w1.shape[0])
+        if self._value_kinds[h] != (self.hidden, self.elem) or self._value_kinds[out][1] != self.elem:
+            raise ValueError("time mixing reads the hidden size and writes the compute dtype")
+        if out_col < 0 or out_col + n > self._value_kinds[out][0]:
+            raise ValueError(f"the result at column {out_col} of a value of {self._value_kinds[out][0]}")
+        self._want(mu, torch.float32, (5, self.hidden), "the blends' mu")
+        self._want(w_rkvg, self.dtype, (4 * n, self.hidden), "the stacked weights of r, k, v and the gate")
+        self._want(w1, self.dtype, (rank, self.hidden), "the decay's inner weight")
+        self._want(w2, self.dtype, (n, rank), "the decay's outer weight")
+        for t, what in ((w0, "the decay's bias"), (bonus, "the bonus"), (norm_weight, "weight of the output norm")):
+            self._want(t, torch.float32, (n,), what)
+        row = heads * head_dim * head_dim + self.hidden
+        self._want(state, torch.float32, (state.shape[0], row), "state")
+        self.op(TIME_MIX, in_=h, out=out, ptrs=[mu, w_rkvg, w1, w2, w0, bonus, norm_weight, state],
+                ints=[heads, head_dim, rank, out_col, row, heads * head_dim * head_dim], floats=[eps, out_scale])
 
     # ----------------------------------------------------------- several residual streams
     def spread_streams(self, streams: int) -> None:

@@ -1,3 +1,3 @@
 """Architecture modules. Importing this package registers every architecture it holds."""
 
-from . import bezurax, gonurax, kifezen, qwen3  # noqa: F401
+from . import bezurax, gonurax, kifezen, qwen3, sevadra  # noqa: F401

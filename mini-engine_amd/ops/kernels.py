@@ -249,6 +249,8 @@ GATE_ACTIVATIONS = {"silu": 1, "gelu_tanh": 2}  # the codes of the kernels' `gat
 # activations that clamp by a limit: the kernels of routed experts take them (with the limit beside the code), the dense
 # products' epilogues do not
 LIMITED_GATE_ACTIVATIONS = {"clamped_sigmoid": 3}
+# activations of a feed-forward without a gate, act(up): codes from 16 on (MeAct in csrc/common.h)
+UNGATED_ACTIVATIONS = {"relu2": 16, "gelu_tanh": 17, "silu": 18}
 
 
 def gate_code(gated, limited: bool = False) -> int:

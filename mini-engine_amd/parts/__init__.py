@@ -1,6 +1,6 @@
 """Parts of a decoder layer. Importing this package registers the built-in kinds."""
 
-from . import attention, decay_state, delta_rule, latent_attention, mlp, norm, pair, rotary, routed_experts  # noqa: F401
+from . import attention, decay_state, delta_rule, latent_attention, mlp, norm, pair, rotary, routed_experts, time_mix  # noqa: F401
 from .base import (
     BLOCK_ARRANGEMENTS,
     FEED_FORWARDS,
@@ -17,7 +17,7 @@ from .base import (
     StateBinding,
     StateNeed,
 )
-from .block import HyperConnectionBlock, ParallelBlock, PreNormBlock, build_block
+from .block import HyperConnectionBlock, ParallelBlock, PreNormBlock, ResultNormBlock, build_block
 from .decoder import Decoder
 
 __all__ = [

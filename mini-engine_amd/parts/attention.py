@@ -23,7 +23,7 @@ import torch
 
 from ..ops import kernels as K
 from ..weights.loader import TensorWant
-from .base import MIXERS, POSITION_ENCODINGS, KVBinding, KVCacheNeed, Mixer
+from .base import MIXERS, POSITION_ENCODINGS, KVBinding, KVCacheNeed, Mixer, PairBinding, StateBinding, StateNeed
 
 MAX_HEAD_DIM = 256
 
@@ -66,11 +66,25 @@ class Attention(Mixer):
             raise ValueError(f"q and k are normed over 'head' or 'projection', not {s.qk_norm_over!r}")
         if (self.values_from_keys or self.pooled_block) and not self.whole:
             raise ValueError("values taken from the keys and pooled blocks are built for q and k normed over their whole projection")
+        # (forms of the attention normed over the whole projection: a short convolution ahead of the norm, a rotation behind it,
+        # bounded scores, a sink of score 0)
+        self.conv_taps = int(getattr(s, "conv_taps", 0))
+        self.softcap = float(getattr(s, "softcap", 0.0) or 0.0)
+        self.unit_sink = bool(getattr(s, "unit_sink", False))
+        if (self.conv_taps or self.softcap or self.unit_sink) and not self.whole:
+            raise ValueError("a short convolution, bounded scores and a sink of score 0 are built for q and k normed over their whole projection")
+        if self.conv_taps < 0 or self.conv_taps > 16 or self.softcap < 0:
+            raise ValueError(f"conv_taps={self.conv_taps} must be in 0..16 and softcap={self.softcap} positive")
         if self.whole:
-            if (s.qk_norm_eps is None or self.position is not None or self.keep_first or self.value_position is not None
+            if (s.qk_norm_eps is None or self.keep_first or self.value_position is not None
                     or self.q_temp is not None or self.gated or s.cache_from is not None or not self.norm_weighted):
-                raise ValueError("attention normed over the whole projection has a weighted norm, no rotation, no kept first keys, "
+                raise ValueError("attention normed over the whole projection has a weighted norm, no kept first keys, "
                                  "no gate, no temperature, and pages of its own")
+            if self.position is not None and (self.pairing != 0 or self.pooled_block or self.values_from_keys):
+                raise ValueError("attention normed over the whole projection is turned in pairs of halves, with a value projection and "
+                                 "without pooled blocks")
+            if self.conv_taps and (self.pooled_block or self.values_from_keys):
+                raise ValueError("a short convolution comes with a value projection and without pooled blocks")
             if self.values_from_keys and self.dv != self.d:
                 raise ValueError(f"values that are the keys have the keys' size {self.d}, not {self.dv}")
             if self.pooled_block < 0 or (self.pooled_block and not s.window):
@@ -90,8 +104,10 @@ class Attention(Mixer):
         self._n = {r: names.get(r, d) for r, d in (("q", "q_proj.weight"), ("k", "k_proj.weight"), ("v", "v_proj.weight"),
                                                     ("o", "o_proj.weight"), ("q_norm", "q_norm.weight"),
                                                     ("k_norm", "k_norm.weight"), ("g", "g_proj.weight"))}
+        self._n.update({r: names.get(r, d) for r, d in (("q_conv", "q_conv.weight"), ("k_conv", "k_conv.weight"), ("v_conv", "v_conv.weight"))})
         self.q_norm_w = self.k_norm_w = None
         self.w_qkv = self.w_o = None
+        self.conv_w = self.sink = None
 
     # ---- weights
     def weight_wants(self, prefix: str) -> dict[str, TensorWant]:
@@ -114,6 +130,9 @@ class Attention(Mixer):
                 wants[f"{prefix}.{n['k_norm']}"] = TensorWant((s.head_dim,), "vector")
         if self.gated:
             wants[f"{prefix}.{n['g']}"] = TensorWant((s.num_heads, s.hidden_size))
+        if self.conv_taps:
+            for role, channels in (("q_conv", s.num_heads * s.head_dim), ("k_conv", s.num_kv_heads * s.head_dim), ("v_conv", s.num_kv_heads * self.dv)):
+                wants[f"{prefix}.{n[role]}"] = TensorWant((channels, self.conv_taps), "vector")
         return wants
 
     def load(self, tensors, prefix: str) -> None:
@@ -133,13 +152,20 @@ class Attention(Mixer):
             self.k_norm_w = tensors.get(f"{prefix}.{n['k_norm']}")
         elif s.qk_norm_eps is not None:  # the norm has no weight: the kernels multiply by ones
             self.q_norm_w = self.k_norm_w = torch.ones(s.head_dim, dtype=torch.float32, device=q.device)
+        if self.conv_taps:  # the three convolutions' weights behind each other, as the channels of [q | k | v] lie
+            self.conv_w = torch.cat([tensors[f"{prefix}.{n[r]}"] for r in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
+        if self.unit_sink:  # a logit of 0 per head in the softmax's denominator
+            self.sink = torch.zeros(s.num_heads, dtype=torch.float32, device=q.device)
 
     # ---- cache
     def cache_need(self):
         if self.spec.cache_from is not None:
             return None
         if self.whole:
-            return KVCacheNeed(self.nkv, self.d, self.spec.window, value_dim=self.dv, pooled_block=self.pooled_block)
+            pages = KVCacheNeed(self.nkv, self.d, self.spec.window, value_dim=self.dv, pooled_block=self.pooled_block)
+            if self.conv_taps > 1:  # the last taps - 1 projections of a sequence, every channel of q, k and v
+                return (pages, StateNeed(((self.conv_taps - 1) * self.input_cols,), torch.float32))
+            return pages
         if self.plain:
             return KVCacheNeed(self.nkv, self.d, self.spec.window)
         return KVCacheNeed(self.nkv, self.d, self.spec.window, value_dim=self.dv, keep_first=self.keep_first)
@@ -229,15 +255,22 @@ class Attention(Mixer):
         ``w_in``), the result goes to the value ``out`` at column ``out_col``, times ``out_scale``."""
         if not self.whole:
             raise NotImplementedError("only attention normed over its whole projection reads and writes at columns of wider values")
+        conv_state = None
+        if isinstance(cache, PairBinding) and isinstance(cache.left, KVBinding) and isinstance(cache.right, StateBinding):
+            cache, conv_state = cache.left, cache.right.state  # pages, and the state rows of the short convolutions
         if not isinstance(cache, KVBinding):
             raise RuntimeError("attention mixer was given no cache")
+        if self.conv_taps > 1 and conv_state is None:
+            raise RuntimeError("attention with a short convolution was given no state rows (it stands alone, not in a pair of mixers)")
         s, b = self.spec, cache
         k_col = col + self.nh * self.d
         program.pooled_attention(
             proj, out, q_col=col, k_col=k_col, v_col=-1 if self.values_from_keys else k_col + self.nkv * self.d, out_col=out_col,
             q_norm=self.q_norm_w, k_norm=self.k_norm_w, k_cache=b.k_cache, v_cache=b.v_cache, k_pool=b.k_pool, v_pool=b.v_pool,
             heads=self.nh, kv_heads=self.nkv, head_dim=self.d, value_dim=self.dv, block_size=b.block_size, window=int(s.window),
-            pooled_block=self.pooled_block, group=b.group, eps=float(s.qk_norm_eps), scale=float(s.scale), out_scale=out_scale)
+            pooled_block=self.pooled_block, group=b.group, eps=float(s.qk_norm_eps), scale=float(s.scale), out_scale=out_scale,
+            rope=None if self.position is None else self.position.tables(program.max_positions), conv=self.conv_w,
+            conv_state=conv_state, sink=self.sink, softcap=self.softcap)
 
     def emit(self, program, h, cache: KVBinding | None = None) -> None:
         s, b = self.spec, cache

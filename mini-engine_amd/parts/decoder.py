@@ -44,6 +44,8 @@ class Decoder:
         wants = {p.embed_name: TensorWant((p.vocab_size, p.hidden_size))}
         for blk in self.blocks:
             wants.update(blk.weight_wants())
+            if callable(getattr(blk, "token_wants", None)):  # an input from the token itself: a slice of a table of the model's
+                wants.update(blk.token_wants(p.vocab_size, int(getattr(p, "token_table_columns", 0))))
         wants.update(self.final_norm.weight_wants(p.final_norm_name))
         if not p.tie_word_embeddings:
             wants[p.head_name] = TensorWant((p.vocab_size, p.hidden_size))

@@ -11,6 +11,12 @@ layer are those of one key/value head. Per step: one product for the queries, th
 three weights are stacked at load time); the latent's norm, the rotation and the page write; the keys' map folded into
 the queries, head by head; attention over the pages (with the sink in the softmax's denominator); the values' map on the
 weighted latents, head by head, times the sigmoid of the head's gate; the output projection.
+
+A position encoding that pairs neighbouring elements (2j with 2j + 1) is served by the kernels that pair halves: the rows of the
+weights that give the turned parts (of the queries, head by head, and of the shared key part) are put into the order ``0, 2, 4, ..,
+1, 3, 5, ..`` when they are loaded. The turned parts only ever meet each other in a score, which no order of their elements changes.
+A layer with ``cache_from`` reads the pages of the layer it names (which orders its shared key part alike) and has no latent
+projection of its own.
 """
 
 from __future__ import annotations
@@ -40,8 +46,10 @@ class LatentAttention(Mixer):
         if not s.output_gate:
             raise ValueError("a latent attention layer has an output gate per head (the ungated form is not built)")
         self.position = POSITION_ENCODINGS.build(s.position, dtype, device)
-        if int(self.position.rotary_dim) != self.r or int(getattr(self.position, "pairing_code", 0)) != 0:
-            raise ValueError("the shared key part is turned over all of its elements, in pairs of halves")
+        if int(self.position.rotary_dim) != self.r:
+            raise ValueError("the shared key part is turned over all of its elements")
+        self.neighbours = int(getattr(self.position, "pairing_code", 0)) == 1
+        self.cache_from = getattr(s, "cache_from", None)
         names = dict(getattr(s, "names", ()) or ())
         self._n = {r: names.get(r, r) for r in ("q", "dkv", "dkv_norm", "uk", "uv", "sink", "g", "o")}
         self.w_in = self.w_o = self.key_map = self.value_map = self.latent_norm = self.sink = None
@@ -51,12 +59,13 @@ class LatentAttention(Mixer):
         s, n = self.spec, self._n
         wants = {
             f"{prefix}.{n['q']}": TensorWant((self.nh * (self.d + self.r), s.hidden_size)),
-            f"{prefix}.{n['dkv']}": TensorWant((self.rank + self.r, s.hidden_size)),
-            f"{prefix}.{n['dkv_norm']}": TensorWant((self.rank,), "vector"),
             f"{prefix}.{n['uk']}": TensorWant((self.nh * self.d, self.rank)),
             f"{prefix}.{n['uv']}": TensorWant((self.nh * self.dv, self.rank)),
             f"{prefix}.{n['o']}": TensorWant((s.hidden_size, self.nh * self.dv)),
         }
+        if self.cache_from is None:
+            wants[f"{prefix}.{n['dkv']}"] = TensorWant((self.rank + self.r, s.hidden_size))
+            wants[f"{prefix}.{n['dkv_norm']}"] = TensorWant((self.rank,), "vector")
         if s.sink:
             wants[f"{prefix}.{n['sink']}"] = TensorWant((self.nh,), "vector")
         if s.output_gate:
@@ -66,7 +75,15 @@ class LatentAttention(Mixer):
     def load(self, tensors, prefix: str) -> None:
         s, n = self.spec, self._n
         q = tensors[f"{prefix}.{n['q']}"]
-        rows = [q, tensors[f"{prefix}.{n['dkv']}"], tensors[f"{prefix}.{n['g']}"]]
+        owns = self.cache_from is None
+        dkv = tensors[f"{prefix}.{n['dkv']}"] if owns else None
+        if self.neighbours:  # the turned parts' rows: evens, then odds (what pairs of neighbours are to the kernels' pairs of halves)
+            order = torch.cat((torch.arange(0, self.r, 2), torch.arange(1, self.r, 2))).to(q.device)
+            q = q.view(self.nh, self.d + self.r, -1)
+            q = torch.cat((q[:, : self.d], q[:, self.d:].index_select(1, order)), dim=1).reshape(self.nh * (self.d + self.r), -1).contiguous()
+            if owns:
+                dkv = torch.cat((dkv[: self.rank], dkv[self.rank:].index_select(0, order)), dim=0).contiguous()
+        rows = [q] + ([dkv] if owns else []) + [tensors[f"{prefix}.{n['g']}"]]
         pad = -sum(t.shape[0] for t in rows) % 8  # rows of zeros: every token's projections then start at a multiple of 16 bytes
         if pad:
             rows.append(torch.zeros((pad, q.shape[1]), dtype=q.dtype, device=q.device))
@@ -75,11 +92,16 @@ class LatentAttention(Mixer):
         # the keys' map per head, transposed: [heads, rank, d] reads a head's query part and gives its image in the latent space
         self.key_map = tensors[f"{prefix}.{n['uk']}"].view(self.nh, self.d, self.rank).transpose(1, 2).contiguous()
         self.value_map = tensors[f"{prefix}.{n['uv']}"].view(self.nh, self.dv, self.rank).contiguous()
-        self.latent_norm = tensors[f"{prefix}.{n['dkv_norm']}"]
+        self.latent_norm = tensors[f"{prefix}.{n['dkv_norm']}"] if owns else torch.ones(self.rank, dtype=torch.float32, device=q.device)
         self.sink = tensors[f"{prefix}.{n['sink']}"] if s.sink else None
 
     # ---- cache
+    def cache_source(self):
+        return self.cache_from
+
     def cache_need(self):
+        if self.cache_from is not None:
+            return None
         # bfloat16 with a key size that the matrix-core attention kernels take and at most 16 heads: those kernels read keys and
         # values of one size, so the value pages hold the whole key (its first `rank` rows are the values that count)
         dk = self.rank + self.r
@@ -99,7 +121,7 @@ class LatentAttention(Mixer):
             proj, latent_norm=self.latent_norm, rope=self.position.tables(program.max_positions), k_cache=b.k_cache,
             v_cache=b.v_cache, key_map=self.key_map, value_map=self.value_map, sink=self.sink, heads=self.nh, head_dim=self.d,
             rotary_dim=self.r, rank=self.rank, value_dim=self.dv, block_size=b.block_size, group=b.group,
-            eps=float(s.norm_eps), scale=float(s.scale))
+            eps=float(s.norm_eps), scale=float(s.scale), writes=self.cache_from is None)
         program.linear_delta(out, self.w_o)
 
 

@@ -47,4 +47,34 @@ class GatedMlp(FeedForward):
         program.linear_delta(act, self.w_down)
 
 
+class ActivatedMlp(FeedForward):
+    """Dense feed-forward without a gate, ``down(act(up(x)))``: a product, the activation as a pass of its own, a product."""
+
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        if spec.activation not in K.UNGATED_ACTIVATIONS:
+            raise ValueError(f"activated_mlp knows the activations {sorted(K.UNGATED_ACTIVATIONS)}, got {spec.activation!r}")
+        names = dict(getattr(spec, "names", ()) or ())
+        self._up, self._down = names.get("up", "up_proj.weight"), names.get("down", "down_proj.weight")
+        self.w_up = self.w_down = None
+
+    def weight_wants(self, prefix: str) -> dict[str, TensorWant]:
+        s = self.spec
+        return {f"{prefix}.{self._up}": TensorWant((s.intermediate_size, s.hidden_size)),
+                f"{prefix}.{self._down}": TensorWant((s.hidden_size, s.intermediate_size))}
+
+    def load(self, tensors, prefix: str) -> None:
+        self.w_up, self.w_down = tensors[f"{prefix}.{self._up}"], tensors[f"{prefix}.{self._down}"]
+
+    def forward(self, h, batch=None):
+        raise NotImplementedError("the ungated feed-forward runs in the step program only")
+
+    def emit(self, program, h) -> None:
+        act = program.activate(program.linear(h, self.w_up), self.spec.activation)
+        program.linear_delta(act, self.w_down)
+
+
 FEED_FORWARDS.register("gated_mlp", GatedMlp)
+FEED_FORWARDS.register("activated_mlp", ActivatedMlp)

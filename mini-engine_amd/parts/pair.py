@@ -7,7 +7,8 @@ write their results, each times its scale (in float32, before the rounding to th
 second product's input. So the pair costs two products a layer, as one mixer does.
 
 A mixer can stand in a pair when it has ``w_in`` (its stacked input weight), ``w_o``, ``input_cols``, ``output_cols`` and
-``emit_projected(program, proj, col, out, out_col, out_scale, cache)``.
+``emit_projected(program, proj, col, out, out_col, out_scale, cache)``. A mixer whose projections do not all read the sublayer's
+input as it is (``reads_input``) has no rows in the stacked product and is handed the input itself, as the keyword ``h``.
 """
 
 from __future__ import annotations
@@ -59,10 +60,15 @@ class PairMixer(Mixer):
         if not isinstance(cache, PairBinding):
             raise RuntimeError("a pair of mixers was given no pair of bindings")
         s = self.spec
+        sides = ((self.left, 0, 0, float(s.left_scale), cache.left),
+                 (self.right, self.left.input_cols, self.left.output_cols, float(s.right_scale), cache.right))
+        reads = any(getattr(m, "reads_input", False) for m in (self.left, self.right))
+        hv = h.value() if reads and hasattr(h, "value") else h  # (the input as a value of its own, where a mixer reads it itself)
         proj = program.linear(h, self.w_in)
         out = program.take(self.left.output_cols + self.right.output_cols)
-        self.left.emit_projected(program, proj, 0, out, 0, float(s.left_scale), cache.left)
-        self.right.emit_projected(program, proj, self.left.input_cols, out, self.left.output_cols, float(s.right_scale), cache.right)
+        for m, col, out_col, scale, binding in sides:
+            extra = {"h": hv} if getattr(m, "reads_input", False) else {}
+            m.emit_projected(program, proj, col, out, out_col, scale, binding, **extra)
         program.linear_delta(out, self.w_o)
 
 

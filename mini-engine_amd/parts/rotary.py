@@ -101,7 +101,54 @@ class YarnRotary(PositionEncoding):
         return self._table
 
 
+class ScaledRotary(PositionEncoding):
+    """Rotation whose slow pairs are slowed by a factor, the fast ones left alone and those between blended by their wavelength
+    (the spec says how). Nothing multiplies the cosines and sines. The table is worked out in double precision on the host and
+    rounded once."""
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        import math
+
+        rd, base = int(spec.rotary_dim), float(spec.theta)
+        if rd <= 0 or rd % 2:
+            raise ValueError(f"rotary_dim must be a positive even number, got {rd}")
+        self.pairing = getattr(spec, "pairing", "halves")
+        if self.pairing not in PAIRINGS:
+            raise ValueError(f"a rotation pairs {sorted(PAIRINGS)}, got {self.pairing!r}")
+        factor, low, high, original = float(spec.factor), float(spec.low), float(spec.high), float(spec.original)
+        if not (factor > 0.0 and original > 0.0 and low > 0.0 and high > low and base > 0.0):
+            raise ValueError("factor, original and low must be positive, high above low")
+        self.rotary_dim, self.pairing_code = rd, PAIRINGS[self.pairing]
+        freq = []
+        for j in range(rd // 2):
+            f = base ** (-2.0 * j / rd)
+            wavelength = 2.0 * math.pi / f
+            if wavelength < original / high:
+                freq.append(f)
+            elif wavelength > original / low:
+                freq.append(f / factor)
+            else:
+                t = (original / wavelength - low) / (high - low)
+                freq.append((1.0 - t) * f / factor + t * f)
+        self.freq = torch.tensor(freq, dtype=torch.float64)
+        self._table: torch.Tensor | None = None
+        self._retired: list[torch.Tensor] = []
+
+    def tables(self, num_positions: int = 1) -> torch.Tensor:
+        if self._table is None or self._table.shape[0] < num_positions:
+            size = 256
+            while size < num_positions:
+                size *= 2
+            if self._table is not None:
+                self._retired.append(self._table)  # a captured graph may still read the smaller table
+            ang = torch.arange(size, dtype=torch.float64)[:, None] * self.freq[None, :]
+            self._table = torch.stack((torch.cos(ang), torch.sin(ang)), dim=1).to(torch.float32).contiguous().to(self.device)
+        return self._table
+
+
 PAIRINGS = {"halves": 0, "neighbours": 1}
 
 POSITION_ENCODINGS.register("rotary", Rotary)
 POSITION_ENCODINGS.register("yarn_rotary", YarnRotary)
+POSITION_ENCODINGS.register("scaled_rotary", ScaledRotary)
