@@ -375,7 +375,8 @@ class Run {
     void* ws = arena_.take((size_t)me_time_mix_workspace(t_, heads, d));
     ok(me_time_shift(bufs_[op.in], (float*)op.p[7], state_row, prev_at, idx(s_.lay.state_slots), idx(s_.lay.item_start), idx(s_.lay.token_item),
                      idx(s_.lay.positions), (const float*)op.p[0], mixes, t_, s_.lay.items, h_, dtype_, stream_));
-    for (int i = 0; i < 4; ++i) product(mixes[i], (const char*)op.p[1] + (size_t)i * n * h_ * elem_, n, h_, 0, dtype_, proj[i]);
+    const void* weights[4] = {op.p[1], op.p[8], op.p[9], op.p[10]};  // r, k, v, gate
+    for (int i = 0; i < 4; ++i) product(mixes[i], weights[i], n, h_, 0, dtype_, proj[i]);
     product(mixes[4], op.p[2], rank, h_, 0, dtype_, z);
     ok(me_time_mix(proj[0], proj[1], proj[2], proj[3], z, op.p[3], (const float*)op.p[4], (const float*)op.p[5], (const float*)op.p[6],
                    (float*)op.p[7], state_row, idx(s_.lay.state_slots), idx(s_.lay.item_start), bufs_[op.out], values_[op.out].cols, (int)op.i[3],

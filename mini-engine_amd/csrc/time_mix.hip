@@ -71,7 +71,7 @@ extern "C" int me_time_shift(const void* h, float* state, long long state_row, l
 }
 
 // decay[t, c] = exp(-exp(sum_j W2[c, j] tanh(z[t, j]) + w0[c])). Grid (tokens), a thread a channel in turns.
-#define TM_MAX_RANK 256
+#define TM_MAX_RANK 1024
 template <typename T>
 __global__ __launch_bounds__(256) void time_decay_kernel(const T* __restrict__ z, const T* __restrict__ W2, const float* __restrict__ w0,
                                                          float* __restrict__ decay, int n, int rank) {

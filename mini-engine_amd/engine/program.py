@@ -432,7 +432,7 @@ class StepProgram:
             raise ValueError(f"{top_k} of {experts + identity_experts} experts a token")
         if scoring not in ROUTER_SCORINGS:
             raise ValueError(f"a router scores by one of {sorted(ROUTER_SCORINGS)}, not {scoring!r}")
-        if num_groups < 1 or experts % num_groups or not 1 <= keep_groups <= num_groups or keep_groups * (experts // num_groups) < top_k:
+        if num_groups < 1 or experts % num_groups or not 1 <= keep_groups <= num_groups or keep_groups * (experts // num_groups) + identity_experts < top_k:
             raise ValueError(f"{experts} experts in {num_groups} groups of which {keep_groups} are kept, {top_k} picks")
         code = UNGATED_ACTIVATIONS[activation] if ungated else gate_code(activation, limited=True)
         self.op(ROUTED_FF, in_=x, ptrs=[router, gate_up, down, shared_gate_up, shared_down, correction],
@@ -579,12 +579,12 @@ class StepProgram:
         self.op(ACTIVATE, in_=x, out=x, ints=[UNGATED_ACTIVATIONS[activation]])
         return x
 
-    def time_mix(self, h: int, out: int, *, out_col: int, mu: torch.Tensor, w_rkvg: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+    def time_mix(self, h: int, out: int, *, out_col: int, mu: torch.Tensor, w_rkvg: tuple, w1: torch.Tensor, w2: torch.Tensor,
                  w0: torch.Tensor, bonus: torch.Tensor, norm_weight: torch.Tensor, state: torch.Tensor, heads: int, head_dim: int,
                  eps: float, out_scale: float = 1.0) -> None:
         """Linear attention with a decay per token and channel and a bonus for the current token, on the value ``h`` ``[tokens, hidden]``
-        (the sublayer's input). ``mu`` float32 ``[5, hidden]`` (the blends of r, k, v, gate, decay with the token before); ``w_rkvg`` ``[4 n,
-        hidden]``, ``w1`` ``[rank, hidden]``, ``w2`` ``[n, rank]`` in the compute dtype (n = heads * head_dim); ``w0``, ``bonus``, ``norm_weight``
+        (the sublayer's input). ``mu`` float32 ``[5, hidden]`` (the blends of r, k, v, gate, decay with the token before); ``w_rkvg`` four weights ``[n,
+        hidden]`` (r, k, v, gate), ``w1`` ``[rank, hidden]``, ``w2`` ``[n, rank]`` in the compute dtype (n = heads * head_dim); ``w0``, ``bonus``, ``norm_weight``
         float32 ``[n]``; ``state`` float32 ``[slots, heads * head_dim^2 + hidden]``. The result (times ``out_scale``) goes to ``out`` at
         ``out_col``."""
         n, rank = heads * head_dim, int(w1.shape[0])
@@ -593,14 +593,15 @@ class StepProgram:
         if out_col < 0 or out_col + n > self._value_kinds[out][0]:
             raise ValueError(f"the result at column {out_col} of a value of {self._value_kinds[out][0]}")
         self._want(mu, torch.float32, (5, self.hidden), "the blends' mu")
-        self._want(w_rkvg, self.dtype, (4 * n, self.hidden), "the stacked weights of r, k, v and the gate")
+        for w in w_rkvg:
+            self._want(w, self.dtype, (n, self.hidden), "a weight of r, k, v or the gate")
         self._want(w1, self.dtype, (rank, self.hidden), "the decay's inner weight")
         self._want(w2, self.dtype, (n, rank), "the decay's outer weight")
         for t, what in ((w0, "the decay's bias"), (bonus, "the bonus"), (norm_weight, "weight of the output norm")):
             self._want(t, torch.float32, (n,), what)
         row = heads * head_dim * head_dim + self.hidden
         self._want(state, torch.float32, (state.shape[0], row), "state")
-        self.op(TIME_MIX, in_=h, out=out, ptrs=[mu, w_rkvg, w1, w2, w0, bonus, norm_weight, state],
+        self.op(TIME_MIX, in_=h, out=out, ptrs=[mu, w_rkvg[0], w1, w2, w0, bonus, norm_weight, state, w_rkvg[1], w_rkvg[2], w_rkvg[3]],
                 ints=[heads, head_dim, rank, out_col, row, heads * head_dim * head_dim], floats=[eps, out_scale])
 
     # ----------------------------------------------------------- several residual streams

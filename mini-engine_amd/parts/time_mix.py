@@ -16,7 +16,7 @@ from ..weights.loader import TensorWant
 from .base import MIXERS, Mixer, StateBinding, StateNeed
 
 MAX_HEAD_DIM = 256  # csrc/time_mix.hip: the scan's widest instance
-MAX_DECAY_RANK = 256  # TM_MAX_RANK
+MAX_DECAY_RANK = 1024  # TM_MAX_RANK
 BLENDS = ("r", "k", "v", "g", "w")  # the order of the rows of mu
 
 
@@ -53,7 +53,7 @@ class TimeMix(Mixer):
     def load(self, tensors, prefix: str) -> None:
         n = self._n
         self.mu = torch.stack([tensors[f"{prefix}.{n['mu_' + b]}"] for b in BLENDS]).contiguous()
-        self.w_rkvg = torch.cat([tensors[f"{prefix}.{n[r]}"] for r in ("r", "k", "v", "g")], dim=0).contiguous()
+        self.w_rkvg = tuple(tensors[f"{prefix}.{n[r]}"].contiguous() for r in ("r", "k", "v", "g"))
         self.w1 = tensors[f"{prefix}.{n['w1']}"].contiguous()
         self.w2 = tensors[f"{prefix}.{n['w2']}"].contiguous()
         self.w_o = tensors[f"{prefix}.{n['o']}"]

@@ -182,19 +182,24 @@ def squared_relu_ff(h, w, p: str):
     return (z * z) @ w[p + ".down"].T
 
 
-def route(h, w, p: str, mlp: dict):
+def route(h, w, p: str, mlp: dict, gaps: list | None = None):
     """(picked [T, top] expert indices, weights [T, top]): softmax over all router outputs, the choice by score plus correction,
-    the weights the scores themselves."""
+    the weights the scores themselves. ``gaps`` collects, per token, how far the last pick's choice score lies above the best
+    score that was not picked (infinite where everything is picked)."""
     top = int(mlp["router"]["top"])
     s = torch.softmax(h @ w[p + ".router"].T, dim=-1)
     choice = s + w[p + ".correction"] if (p + ".correction") in w else s
-    picked = torch.topk(choice, top, dim=-1).indices
+    ranked = torch.sort(choice, dim=-1, descending=True)
+    picked = ranked.indices[:, :top]
+    if gaps is not None:
+        gaps.append(ranked.values[:, top - 1] - ranked.values[:, top] if choice.shape[1] > top
+                    else torch.full((h.shape[0],), math.inf, dtype=h.dtype))
     return picked, torch.gather(s, 1, picked)
 
 
-def routed_ff(h, w, p: str, mlp: dict):
+def routed_ff(h, w, p: str, mlp: dict, gaps: list | None = None):
     experts = int(mlp["router"]["experts"])
-    picked, weights = route(h, w, p, mlp)
+    picked, weights = route(h, w, p, mlp, gaps)
     out = torch.zeros_like(h)
     for i in range(h.shape[0]):
         for e, wt in zip(picked[i].tolist(), weights[i]):
@@ -215,8 +220,11 @@ def token_side_input(x, tokens, w, cfg: dict, i: int, eps: float):
     return rms_norm(y, w[f"l{i}.side.norm"], eps)
 
 
-def forward(cfg: dict, weights: dict, tokens, return_layers: bool = False):
-    """Logits [T, vocab] of one sequence (float64); with ``return_layers`` also the stream after every layer."""
+def forward(cfg: dict, weights: dict, tokens, return_layers: bool = False, router_gaps: list | None = None, reads=None):
+    """Logits [T, vocab] of one sequence (float64); with ``return_layers`` also the stream after every layer. ``router_gaps``
+    collects what :func:`route` says of every routed layer. ``reads`` (a function of the stream, or None) stands between the
+    stream and every sublayer that reads it: what a rounding there does to the logits says how well a row bears roundings."""
+    reads = reads or (lambda z: z)
     w = {k: (v.to(F64) if v.is_floating_point() else v) for k, v in weights.items()}
     eps = float(cfg["norm"]["eps"])
     tokens = torch.as_tensor(tokens, dtype=torch.long)
@@ -225,26 +233,28 @@ def forward(cfg: dict, weights: dict, tokens, return_layers: bool = False):
     after = []
     for i, layer in enumerate(cfg["layers"]):
         m, kind, p = layer["mixer"], layer["type"], f"l{i}.mix"
+        h = reads(x)
         if kind == "attention":
-            y = attention_mixer(x, w, p, m, eps)
+            y = attention_mixer(h, w, p, m, eps)
         elif kind == "parallel":
-            y = float(m["left_scale"]) * capped_sink_attention(x, w, p + ".left", m["left"], eps) \
-                + float(m["right_scale"]) * time_mixing(x, w, p + ".right", m["right"], eps)
+            y = float(m["left_scale"]) * capped_sink_attention(h, w, p + ".left", m["left"], eps) \
+                + float(m["right_scale"]) * time_mixing(h, w, p + ".right", m["right"], eps)
         elif kind == "latent_attention":
             src = m.get("kv_from")
             if src is None:
-                latents[i] = latent_projection(x, w, p, m, eps)
+                latents[i] = latent_projection(h, w, p, m, eps)
                 src = i
-            y = latent_attention(x, w, p, m, latents[int(src)], eps)
+            y = latent_attention(h, w, p, m, latents[int(src)], eps)
         else:
             raise ValueError(kind)
         x = x + rms_norm(y, w[f"l{i}.norm1"], eps)
         mlp = layer.get("mlp")
         if mlp is not None:
-            y = squared_relu_ff(x, w, f"l{i}.mlp") if mlp["kind"] == "dense" else routed_ff(x, w, f"l{i}.mlp", mlp)
+            h = reads(x)
+            y = squared_relu_ff(h, w, f"l{i}.mlp") if mlp["kind"] == "dense" else routed_ff(h, w, f"l{i}.mlp", mlp, router_gaps)
             x = x + rms_norm(y, w[f"l{i}.norm2"], eps)
         if cfg.get("token_side"):
-            x = x + token_side_input(x, tokens, w, cfg, i, eps)
+            x = x + token_side_input(reads(x), tokens, w, cfg, i, eps)
         after.append(x.clone())
     logits = rms_norm(x, w["final.norm"], eps) @ w["embed"].T
     return (logits, after) if return_layers else logits
