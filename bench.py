@@ -408,14 +408,44 @@ def bezurax_config(size: str):
                                     "norm": {"eps": 1e-6, "groups": 2}, "layers": order})
 
 
+def sevadra_config(size: str):
+    """Eight layers whose norms sit on the sublayers' results, each with an input of 64 elements from the token itself; twice the
+    run latent attention (16 heads of 128 + 64 turned, values of 128, a latent of 192: a cached key of 256) with a dense feed-forward;
+    a pair of mixers (left: 16 heads of 128 on 8 key/value heads, bounded scores and a sink; right: time mixing over heads of 64 that
+    fill the width, a decay of inner size 64); attention with short convolutions of 4 taps (16 heads of 128 on 8 key/value heads,
+    slowed rotation); latent attention over the first layer's latents. But for the first, the feed-forwards are 16 routed experts
+    without a gate of two thirds of the size's feed-forward (as many weights as a gated expert of a third), 4 identity experts, two a
+    token, and a shared expert of the same size."""
+    from mini_engine_amd.models.sevadra import SevadraConfig
+
+    z = DESIGN_SIZES[size]
+    ff = 2 * z["ff"] // 3
+    moe = {"kind": "moe", "expert": {"ff": ff // 2}, "shared": {"ff": ff // 2}, "router": {"experts": 16, "identity": 4, "top": 2}}
+    rot = {"base": 5e5, "dims": 64}
+    lat = {"heads": z["heads"], "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "scale": 192 ** -0.5, "rot": rot}
+    left = {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0}
+    right = {"heads": z["width"] // 64, "dim": 64, "decay_rank": 64}
+    att = {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 4,
+           "rot": {"base": 1e4, "dims": 128, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    order = []
+    for first in range(0, DESIGN_LAYERS, 4):
+        order += [{"type": "latent_attention", "mixer": lat, "mlp": {"kind": "dense", "ff": z["ff"] * 3 // 2}},
+                  {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 0.8, "right_scale": 0.9}, "mlp": moe},
+                  {"type": "attention", "mixer": att, "mlp": moe},
+                  {"type": "latent_attention", "mixer": dict(lat, kv_from=first), "mlp": moe}]
+    return SevadraConfig.from_dict({"architecture": "Sevadra", "vocab": DESIGN_VOCAB, "width": z["width"], "norm": {"eps": 1e-6},
+                                    "token_side": {"dim": 64}, "layers": order})
+
+
 # design -> (architecture, its configuration at a size, the model beside it: "qwen3" or another design of this table)
 DESIGNS = {"gonurax": ("Gonurax", gonurax_config, "qwen3"), "kifezen": ("Kifezen", kifezen_config, "qwen3"),
-           "bezurax": ("Bezurax", bezurax_config, "gonurax")}
+           "bezurax": ("Bezurax", bezurax_config, "gonurax"), "sevadra": ("Sevadra", sevadra_config, "bezurax")}
 
 
 def design_line(args) -> dict:
     """Prefill and decode throughput of a design beside the model closest to it (the Qwen3 dense design for Gonurax and Kifezen,
-    the Gonurax design, which has windowed attention beside recurrent layers, for Bezurax) at equal layer sizes (random
+    the Gonurax design, which has windowed attention beside recurrent layers, for Bezurax; the Bezurax design, which has a pair of
+    mixers with a recurrent one and routed experts with a shared one, for Sevadra) at equal layer sizes (random
     weights, eight layers): a 2,048-token prompt, and decode steps at batch 1, 8 and 64 behind a context of 2,304."""
     from mini_engine_amd.models.qwen3 import Qwen3Config
 
@@ -471,7 +501,7 @@ def main() -> int:
     ap.add_argument("--skip-prefill", action="store_true", help="profiling aid: do not measure the prefill")
     ap.add_argument("--skip-extras", action="store_true",
                     help="profiling aid: only the decode steps and the prefill (no serving workloads, no float32 point, no probes)")
-    ap.add_argument("--design", default="", choices=["", "gonurax", "kifezen", "bezurax"],
+    ap.add_argument("--design", default="", choices=["", "gonurax", "kifezen", "bezurax", "sevadra"],
                     help="instead of the default workload: this design beside the model closest to it at equal layer sizes")
     ap.add_argument("--design-sizes", default="1024,2048", help="widths of --design to measure, comma separated")
     ap.add_argument("--design-batches", default="1,8,64", help="decode batch sizes of --design, comma separated")

@@ -148,7 +148,7 @@ __global__ __launch_bounds__(1024) void routed_route_kernel(const T* __restrict_
   // sorted as routed_sort_kernel leaves them for tiles of one row).
   if (plan && lane < top) {
     const int pair = t * top + lane;
-    plan[1 + 3 * pair] = mine_e;
+    plan[1 + 3 * pair] = mine_e < E_real ? mine_e : 0;  // (never an index beyond the experts that have tensors)
     plan[2 + 3 * pair] = pair;
     plan[3 + 3 * pair] = mine_e < E_real ? 1 : 0;  // (an identity expert: a tile of no rows)
     sorted[pair] = pair;
@@ -193,6 +193,7 @@ __global__ __launch_bounds__(256) void routed_gate_up_kernel(const T* __restrict
   const int tile = blockIdx.x;
   if (tile >= plan[0]) return;
   const int e = plan[1 + 3 * tile], begin = plan[2 + 3 * tile], rows = plan[3 + 3 * tile];
+  if (rows <= 0) return;  // (the pair of an identity expert, where the router wrote the list itself: no weights to read)
   const int c0 = blockIdx.y * TP_COLS, cols = min(TP_COLS, ff - c0);
   auto row_ptr = [&](int i) { return h + (size_t)(sorted[begin + i] / top) * hidden; };
   const bool ungated = act_is_ungated(act);  // W_gu is [E, ff, hidden] then: up rows alone
@@ -220,6 +221,7 @@ __global__ __launch_bounds__(256) void routed_down_kernel(const T* __restrict__ 
   const int tile = blockIdx.x;
   if (tile >= plan[0]) return;
   const int e = plan[1 + 3 * tile], begin = plan[2 + 3 * tile], rows = plan[3 + 3 * tile];
+  if (rows <= 0) return;  // (the pair of an identity expert, where the router wrote the list itself: no weights to read)
   const int c0 = blockIdx.y * TP_COLS, cols = min(TP_COLS, hidden - c0);
   float acc[4];
   tile_product<T>([&](int i) { return acts + (size_t)(begin + i) * ff; }, rows, W_down + ((size_t)e * hidden + c0) * ff, cols, ff,
@@ -250,6 +252,7 @@ __global__ __launch_bounds__(256) void routed_tile_mfma_kernel(const bf16_t* __r
   const int tile = blockIdx.x;
   if (tile >= plan[0]) return;
   const int e = plan[1 + 3 * tile], begin = plan[2 + 3 * tile], rows = plan[3 + 3 * tile];
+  if (rows <= 0) return;  // (the pair of an identity expert, where the router wrote the list itself: no weights to read)
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1), r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.y * 64 + wave * 16;
   if (n0 >= N) return;
@@ -302,6 +305,7 @@ __global__ __launch_bounds__(256) void routed_tile_ksplit_kernel(const bf16_t* _
   const int tile = blockIdx.x;
   if (tile >= plan[0]) return;
   const int e = plan[1 + 3 * tile], begin = plan[2 + 3 * tile], rows = plan[3 + 3 * tile];
+  if (rows <= 0) return;  // (the pair of an identity expert, where the router wrote the list itself: no weights to read)
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1), r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.y * 16;
   const bf16_t* w0 = n0 + r < N ? W + ((size_t)e * ACCS * N + n0 + r) * K : nullptr;
