@@ -95,10 +95,18 @@ __device__ __forceinline__ void load_tile(KvTile<D>& t, const bf16_t* __restrict
     t.vf[dt] = *reinterpret_cast<const short4_t*>(vbase + (size_t)(dt * 16 + r) * bs + g * 4);
 }
 
+// Bounded scores, cap * tanh(score * scale / cap): the kernels turn a raw score s into tanh(s * cap_c1) with cap_c1 = scale / cap
+// right behind the product that gives it, and the host hands them cap * log2(e) as the scale of what follows. tanh rises with its
+// argument, so a maximum taken over transformed scores is the transformed maximum, as the kernels' running maxima assume.
+__device__ __forceinline__ float bounded_score(float s, float cap_c1) {
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(fast_exp2(s * (cap_c1 * 2.885390081777927f)) + 1.f);  // tanh(x) = 1 - 2 / (e^(2x) + 1)
+}
+
 template <int D, int NB>
 __device__ __forceinline__ void compute_tile(const KvTile<D>& t, int key0, int lo, const int (&qpos)[NB],
                                              bool need_mask, const Frag8 (&qf)[NB][D / 32], float scale_log2,
-                                             float (&m)[NB], float (&lsum)[NB], float4_t (&acc)[NB][D / 16], int keep_first = 0) {
+                                             float (&m)[NB], float (&lsum)[NB], float4_t (&acc)[NB][D / 16], int keep_first = 0,
+                                             float cap_c1 = 0.f) {
   const int lane = threadIdx.x & (ME_WAVE - 1);
   const int g = lane >> 4;
   short4_t pf[NB];
@@ -113,7 +121,7 @@ __device__ __forceinline__ void compute_tile(const KvTile<D>& t, int key0, int l
     float sv[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      sv[i] = s[i] * scale_log2;
+      sv[i] = (cap_c1 > 0.f ? bounded_score(s[i], cap_c1) : s[i]) * scale_log2;
       if (need_mask) {
         const int key = key0 + g * 4 + i;
         if ((key < lo && key >= keep_first) || key > qpos[nb]) sv[i] = -INFINITY;
@@ -180,6 +188,7 @@ struct DecodeFusedArgs {
   long long out_row = 0;
   int out_col = 0;
   float out_scale = 1.f;
+  float cap_c1 = 0.f;  // > 0: scores are bounded (bounded_score)
 };
 
 // Tiles of a split from which on a wave fetches one tile at a time, whatever DEPTH says: with five tiles and more of its own
@@ -374,7 +383,7 @@ __device__ __forceinline__ void attention_decode_body(
       const int key0 = key_at(place);
       const int qpos[1] = {of_pool ? pooled - 1 : ctx - 1};
       compute_tile<D, 1>(tile, key0, of_pool ? 0 : lo, qpos, of_pool ? key0 + 16 > pooled : (place < lo || place + 16 > ctx), qf,
-                         scale_log2, m, lsum, acc, of_pool ? 0 : keep_first);
+                         scale_log2, m, lsum, acc, of_pool ? 0 : keep_first, fa.cap_c1);
     };
     if (!early) fetch(t[0], begin);
     // DEPTH tiles in flight per wave: tile i + DEPTH - 1 is requested before the products of tile i. Short
@@ -725,6 +734,25 @@ extern "C" int me_attention_decode_bf16_pooled(const void* q, const void* k_cach
                        nullptr, &pool);
 }
 
+// As me_attention_decode_bf16, with the result placed (rows out_row elements apart, 0: nh * d; from column out_col on; times
+// out_scale), an optional sink (float32 [nh] logits that count once in the denominator) and, with softcap > 0, scores bounded by
+// softcap * tanh(score * scale / softcap).
+extern "C" int me_attention_decode_bf16_placed(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
+                                               const int* block_table, int table_width, void* out, long long out_row, int out_col,
+                                               float out_scale, float* part_o, float* part_ml, int items, int nh, int nkv, int d, int bs,
+                                               int window, float scale, float softcap, const float* sink, int split_keys, int num_splits,
+                                               int max_ctx, const int* live_items, int full_splits, int waves_wanted,
+                                               const int* step_flags, hipStream_t stream) {
+  DecodeFusedArgs place{};
+  place.out_row = out_row;
+  place.out_col = out_col;
+  place.out_scale = out_scale;
+  place.cap_c1 = softcap > 0.f ? scale / softcap : 0.f;
+  return decode_common(q, k_cache, v_cache, item_ctx, block_table, table_width, out, part_o, part_ml, items, nh, nkv, d, bs, window,
+                       scale, split_keys, num_splits, max_ctx, nullptr, live_items, full_splits, waves_wanted, step_flags, stream, 0,
+                       sink, &place);
+}
+
 extern "C" int me_attention_decode_bf16_sink(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
                                              const int* block_table, int table_width, void* out, float* part_o,
                                              float* part_ml, int items, int nh, int nkv, int d, int bs, const float* sink,
@@ -786,7 +814,8 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
                          int waves_wanted, const int* step_flags, hipStream_t stream, int keep_first, const float* sink,
                          const DecodeFusedArgs* pool) {
   if (items <= 0) return 0;
-  if (pool && (fused || keep_first > 0 || sink || window <= 0 || pool->pool_block < 0 || (pool->pool_block > 0 && (!pool->k_pool || !pool->v_pool))))
+  if (pool && (fused || keep_first > 0 || pool->pool_block < 0 ||
+               (pool->pool_block > 0 && (sink || window <= 0 || pool->cap_c1 > 0.f || !pool->k_pool || !pool->v_pool))))
     return me_fail("me_attention_decode_bf16: pooled blocks of %d keys need a window, pages of their own, the unfused form, no kept "
                    "first keys and no sink", pool->pool_block);
   if (pool && (pool->out_col < 0 || (pool->out_row > 0 && pool->out_col + (long long)nh * d > pool->out_row) || (pool->out_row > 0 && !out)))
@@ -826,7 +855,8 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   // do not take it up to 4%.)
   const long long kv_bytes = (long long)items * max_ctx * nkv * d * 4;
   const int streamed = kv_bytes >= (256ll << 20) && (block_waves == 1 || blocks >= cus);
-  const float sl = scale * LOG2E;
+  // (bounded scores: the kernel turns a raw score into tanh(score * scale / cap); what follows is scaled by cap * log2(e))
+  const float sl = pool && pool->cap_c1 > 0.f ? scale / pool->cap_c1 * LOG2E : scale * LOG2E;
   const bf16_t *qq = (const bf16_t*)q, *kc = (const bf16_t*)k_cache, *vc = (const bf16_t*)v_cache;
 #define ME_DECODE_CASE(DD)                                                                                      \
   case DD:                                                                                                      \
@@ -1029,7 +1059,7 @@ template <int D, int NB, bool MASK>
 __device__ __forceinline__ void pf_softmax_pv64(const bf16_t* __restrict__ vs, int key_base, int r, int g,
                                                 const float4_t (&s)[NB][4], const int (&qpos)[NB], const int (&lo_col)[NB],
                                                 float scale_log2, float (&m)[NB], float (&lsum)[NB],
-                                                float4_t (&acc)[NB][D / 16], int keep_first) {
+                                                float4_t (&acc)[NB][D / 16], int keep_first, float cap_c1 = 0.f) {
   using L = PrefillLds<D>;
   bf16x8_t pf[NB][2];
 #pragma unroll
@@ -1039,6 +1069,10 @@ __device__ __forceinline__ void pf_softmax_pv64(const bf16_t* __restrict__ vs, i
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) sv[t * 4 + i] = s[nb][t][i];
+    if (cap_c1 > 0.f) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sv[i] = bounded_score(sv[i], cap_c1);
+    }
     if (MASK) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
@@ -1114,6 +1148,7 @@ struct PrefillPool {
   long long out_row;
   int out_col;
   float out_scale;
+  float cap_c1 = 0.f;  // > 0: scores are bounded (bounded_score)
 };
 
 struct PrefillWork {
@@ -1219,9 +1254,9 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     if (active) {
       const bool need_mask = key0 + PF_KT - 1 > wave_min_pos || win > 0;
       if (need_mask)
-        pf_softmax_pv64<D, NB, true>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc, keep);
+        pf_softmax_pv64<D, NB, true>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc, keep, pool.cap_c1);
       else
-        pf_softmax_pv64<D, NB, false>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc, keep);
+        pf_softmax_pv64<D, NB, false>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc, keep, pool.cap_c1);
     }
     __syncthreads();
   }
@@ -1358,7 +1393,7 @@ static int prefill_common(const void* q, const void* k_cache, const void* v_cach
   const int num_work = num_bundles;
   PrefillPool pool{nullptr, nullptr, 0, 0, 0, 1.f};
   if (pooled) pool = *pooled;
-  if (pool.block < 0 || (pool.block > 0 && (window <= 0 || keep_first > 0 || sink || !pool.k_pool || !pool.v_pool)))
+  if (pool.block < 0 || (pool.block > 0 && (window <= 0 || keep_first > 0 || sink || pool.cap_c1 > 0.f || !pool.k_pool || !pool.v_pool)))
     return me_fail("me_attention_prefill_bf16: pooled blocks of %d keys need a window, pages of their own, no kept first keys and no "
                    "sink", pool.block);
   if (pool.out_col < 0 || (pool.out_row > 0 && pool.out_col + (long long)nh * d > pool.out_row) || ((pool.out_row | pool.out_col) & 3))
@@ -1382,7 +1417,8 @@ static int prefill_common(const void* q, const void* k_cache, const void* v_cach
     return me_fail("me_attention_prefill_bf16: %d query columns per block (%d or %d)", columns, PF_COLUMNS_NARROW, PF_COLUMNS_WIDE);
   const bool wide = columns == PF_COLUMNS_WIDE;
   const int tpb = columns / group;
-  const float sl = scale * LOG2E;
+  // (bounded scores: the kernel turns a raw score into tanh(score * scale / cap); what follows is scaled by cap * log2(e))
+  const float sl = pool.cap_c1 > 0.f ? scale / pool.cap_c1 * LOG2E : scale * LOG2E;
   int bs_shift = 0;
   while ((1 << bs_shift) < bs) ++bs_shift;
   dim3 grid((unsigned)num_work * nkv);
@@ -1439,6 +1475,20 @@ extern "C" int me_attention_prefill_bf16_pooled(const void* q, const void* k_cac
   return prefill_common(q, k_cache, v_cache, num_items, block_table, table_width, out, work, bundle_first, num_bundles, part_o,
                         part_ml, token_chunks, max_chunks, num_tokens, nh, nkv, d, bs, window, 0, scale, columns, nullptr, stream,
                         &pool);
+}
+
+// As me_attention_prefill_bf16, with the result placed (rows out_row elements apart, 0: nh * d; from column out_col on; times
+// out_scale), an optional sink and, with softcap > 0, scores bounded by softcap * tanh(score * scale / softcap).
+extern "C" int me_attention_prefill_bf16_placed(const void* q, const void* k_cache, const void* v_cache, int num_items,
+                                                const int* block_table, int table_width, void* out, long long out_row, int out_col,
+                                                float out_scale, const int* work, const int* bundle_first, int num_bundles,
+                                                float* part_o, float* part_ml, const int* token_chunks, int max_chunks, int num_tokens,
+                                                int nh, int nkv, int d, int bs, int window, float scale, float softcap,
+                                                const float* sink, int columns, hipStream_t stream) {
+  PrefillPool place{nullptr, nullptr, 0, out_row, out_col, out_scale};
+  place.cap_c1 = softcap > 0.f ? scale / softcap : 0.f;
+  return prefill_common(q, k_cache, v_cache, num_items, block_table, table_width, out, work, bundle_first, num_bundles, part_o,
+                        part_ml, token_chunks, max_chunks, num_tokens, nh, nkv, d, bs, window, 0, scale, columns, sink, stream, &place);
 }
 
 // All keys visible, with a sink (see prefill_common).

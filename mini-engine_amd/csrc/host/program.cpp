@@ -171,9 +171,9 @@ bool attention_takes_tiled_prefill(const Op& op, int dtype) {
 // one size that the kernels are built for, up to 16 heads to a key/value head, results at rows and a column that are multiples of 4.
 bool pooled_takes_matrix_cores(const Op& op, int dtype, long long out_row) {
   const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2], dv = (int)op.i[3], bs = (int)op.i[4];
-  if (op.p[9] || op.f[3] > 0.f) return false;  // (a sink without a value, bounded scores: the kernel that takes every form)
-  return dtype == kBF16 && dv == d && op.i[5] > 0 && me_attention_mfma_supported(d, bs) && nh / nkv <= 16 && out_row % 4 == 0 &&
-         op.i[11] % 4 == 0;
+  // (pooled blocks lie before a window; without them the kernels take every window, none, a sink and bounded scores)
+  return dtype == kBF16 && dv == d && (op.i[5] > 0 || op.i[6] == 0) && me_attention_mfma_supported(d, bs) && nh / nkv <= 16 &&
+         out_row % 4 == 0 && op.i[11] % 4 == 0;
 }
 
 int groups_of(int64_t v) { return v > 1 ? (int)v : 1; }
@@ -892,10 +892,16 @@ class Run {
       const SplitPlan sp = split_plan(items, nkv * ((nh / nkv + 15) / 16), s_.max_ctx, s_.least_live, idx(s_.lay.live_items));
       float* part_o = (float*)arena_.take((size_t)items * nh * sp.num_splits * d * 4);
       float* part_ml = (float*)arena_.take((size_t)items * nh * sp.num_splits * 2 * 4);
-      ok(me_attention_decode_bf16_pooled(q, op.p[2], op.p[3], op.p[4], op.p[5], pool, idx(s_.lay.item_ctx), table, width, bufs_[op.out],
-                                         out_row, (int)op.i[11], out_scale, part_o, part_ml, items, nh, nkv, d, bs, window, op.f[1],
-                                         sp.split_keys, sp.num_splits, s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves,
-                                         idx(s_.lay.live_items) + 1, stream_));
+      if (pool > 0)
+        ok(me_attention_decode_bf16_pooled(q, op.p[2], op.p[3], op.p[4], op.p[5], pool, idx(s_.lay.item_ctx), table, width, bufs_[op.out],
+                                           out_row, (int)op.i[11], out_scale, part_o, part_ml, items, nh, nkv, d, bs, window, op.f[1],
+                                           sp.split_keys, sp.num_splits, s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves,
+                                           idx(s_.lay.live_items) + 1, stream_));
+      else
+        ok(me_attention_decode_bf16_placed(q, op.p[2], op.p[3], idx(s_.lay.item_ctx), table, width, bufs_[op.out], out_row, (int)op.i[11],
+                                           out_scale, part_o, part_ml, items, nh, nkv, d, bs, window, op.f[1], softcap, sink, sp.split_keys,
+                                           sp.num_splits, s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves, idx(s_.lay.live_items) + 1,
+                                           stream_));
       return;
     }
     if (pooled_takes_matrix_cores(op, dtype_, out_row)) {
@@ -908,10 +914,16 @@ class Run {
         part_o = (float*)arena_.take((size_t)t_ * nh * p.max_chunks * d * 4);
         part_ml = (float*)arena_.take((size_t)t_ * nh * p.max_chunks * 2 * 4);
       }
-      ok(me_attention_prefill_bf16_pooled(q, op.p[2], op.p[3], op.p[4], op.p[5], pool, s_.lay.items, table, width, bufs_[op.out], out_row,
-                                          (int)op.i[11], out_scale, idx(p.work), idx(p.bundle_first), p.bundles, part_o, part_ml,
-                                          p.token_chunks >= 0 ? idx(p.token_chunks) : nullptr, p.max_chunks, t_, nh, nkv, d, bs, window,
-                                          op.f[1], p.columns, stream_));
+      if (pool > 0)
+        ok(me_attention_prefill_bf16_pooled(q, op.p[2], op.p[3], op.p[4], op.p[5], pool, s_.lay.items, table, width, bufs_[op.out], out_row,
+                                            (int)op.i[11], out_scale, idx(p.work), idx(p.bundle_first), p.bundles, part_o, part_ml,
+                                            p.token_chunks >= 0 ? idx(p.token_chunks) : nullptr, p.max_chunks, t_, nh, nkv, d, bs, window,
+                                            op.f[1], p.columns, stream_));
+      else
+        ok(me_attention_prefill_bf16_placed(q, op.p[2], op.p[3], s_.lay.items, table, width, bufs_[op.out], out_row, (int)op.i[11], out_scale,
+                                            idx(p.work), idx(p.bundle_first), p.bundles, part_o, part_ml,
+                                            p.token_chunks >= 0 ? idx(p.token_chunks) : nullptr, p.max_chunks, t_, nh, nkv, d, bs, window,
+                                            op.f[1], softcap, sink, p.columns, stream_));
       return;
     }
     ok(me_attention_general_capped(q, op.p[2], op.p[3], idx(s_.lay.positions), idx(s_.lay.token_item), table, width, bufs_[op.out], t_, nh,

@@ -229,4 +229,14 @@ int me_time_mix(const void* r, const void* k, const void* v, const void* gate, c
                 const float* bonus, const float* norm_w, float* state, long long state_row, const int* state_slots, const int* item_start,
                 void* out, long long out_row, int out_col, float out_scale, int num_tokens, int items, int heads, int d, int rank, float eps,
                 int dtype, void* workspace, hipStream_t stream);
+int me_attention_decode_bf16_placed(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx, const int* block_table,
+                                    int table_width, void* out, long long out_row, int out_col, float out_scale, float* part_o,
+                                    float* part_ml, int items, int nh, int nkv, int d, int bs, int window, float scale, float softcap,
+                                    const float* sink, int split_keys, int num_splits, int max_ctx, const int* live_items, int full_splits,
+                                    int waves_wanted, const int* step_flags, hipStream_t stream);
+int me_attention_prefill_bf16_placed(const void* q, const void* k_cache, const void* v_cache, int num_items, const int* block_table,
+                                     int table_width, void* out, long long out_row, int out_col, float out_scale, const int* work,
+                                     const int* bundle_first, int num_bundles, float* part_o, float* part_ml, const int* token_chunks,
+                                     int max_chunks, int num_tokens, int nh, int nkv, int d, int bs, int window, float scale, float softcap,
+                                     const float* sink, int columns, hipStream_t stream);
 }

@@ -139,6 +139,117 @@ __global__ __launch_bounds__(64) void time_scan_kernel(const T* __restrict__ r, 
   }
 }
 
+// The scan for heads of D = 32, 64 or 128 elements, a block per (item, head) and a wave per 16 value channels of it. The block walks the
+// item's tokens in chunks of TS_CHUNK: all threads fetch a chunk's r, k, v and decays together (16 bytes a load, every load of the chunk
+// in flight at once, and the next chunk's asked for before this one is worked on) and lay them out in LDS as float32; then every wave
+// walks the chunk's tokens out of LDS. The sums are those of time_scan_kernel, in its order: a token's result is the same bits
+// whichever of the two kernels serves it.
+#define TS_CHUNK 32
+template <typename T>
+struct TsVec;  // eight consecutive elements of a row
+template <>
+struct TsVec<bf16_t> {
+  uint4 raw;
+  __device__ __forceinline__ void load(const bf16_t* p) { raw = *reinterpret_cast<const uint4*>(p); }
+  __device__ __forceinline__ void zero() { raw = make_uint4(0, 0, 0, 0); }
+  __device__ __forceinline__ void store(float* dst) const {
+    const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      dst[2 * i] = __uint_as_float(w4[i] << 16);
+      dst[2 * i + 1] = __uint_as_float(w4[i] & 0xffff0000u);
+    }
+  }
+};
+template <>
+struct TsVec<float> {
+  float4 a, b;
+  __device__ __forceinline__ void load(const float* p) {
+    a = *reinterpret_cast<const float4*>(p);
+    b = *reinterpret_cast<const float4*>(p + 4);
+  }
+  __device__ __forceinline__ void zero() { a = b = make_float4(0.f, 0.f, 0.f, 0.f); }
+  __device__ __forceinline__ void store(float* dst) const {
+    *reinterpret_cast<float4*>(dst) = a;
+    *reinterpret_cast<float4*>(dst + 4) = b;
+  }
+};
+
+template <typename T, int D>
+__global__ __launch_bounds__(4 * D) void time_scan_chunked_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v,
+                                                                 const float* __restrict__ decay, const float* __restrict__ bonus,
+                                                                 float* __restrict__ state, long long state_row,
+                                                                 const int* __restrict__ state_slots, const int* __restrict__ item_start,
+                                                                 float* __restrict__ o, int heads) {
+  constexpr int RPL = D / 4, VPR = D / 8;  // rows of S a lane holds; vectors of eight elements a row
+  __shared__ __attribute__((aligned(16))) float lr[TS_CHUNK][D], lk[TS_CHUNK][D], lv[TS_CHUNK][D], lw[TS_CHUNK][D];
+  const int item = blockIdx.x / heads, head = blockIdx.x % heads;
+  const int tid = threadIdx.x, wave = tid / ME_WAVE, lane = tid & (ME_WAVE - 1);
+  const int p = lane >> 4, c = wave * 16 + (lane & 15), i0 = p * RPL;
+  const int first = item_start[item], end = item_start[item + 1];
+  const int n = heads * D;
+  float* S = state + (size_t)state_slots[item] * state_row + (size_t)head * D * D;
+  float s[RPL], u[RPL];
+#pragma unroll
+  for (int a = 0; a < RPL; ++a) {
+    s[a] = S[(size_t)(i0 + a) * D + c];
+    u[a] = bonus[head * D + i0 + a];
+  }
+  // this thread's vector of a chunk: token tid / VPR of the chunk, elements 8 (tid % VPR) .. + 7 of the head's row
+  const int vt = tid / VPR, ve = 8 * (tid % VPR);
+  TsVec<T> fr, fk, fv;
+  float4 fw0, fw1;
+  auto fetch = [&](int t0) {
+    const int t = t0 + vt;
+    if (t < end) {
+      const size_t at = (size_t)t * n + head * D + ve;
+      fr.load(r + at);
+      fk.load(k + at);
+      fv.load(v + at);
+      fw0 = *reinterpret_cast<const float4*>(decay + at);
+      fw1 = *reinterpret_cast<const float4*>(decay + at + 4);
+    } else {
+      fr.zero(), fk.zero(), fv.zero();
+      fw0 = fw1 = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  };
+  if (first < end) fetch(first);
+  for (int t0 = first; t0 < end; t0 += TS_CHUNK) {
+    __syncthreads();  // the chunk before is worked off
+    fr.store(&lr[vt][ve]);
+    fk.store(&lk[vt][ve]);
+    fv.store(&lv[vt][ve]);
+    *reinterpret_cast<float4*>(&lw[vt][ve]) = fw0;
+    *reinterpret_cast<float4*>(&lw[vt][ve + 4]) = fw1;
+    __syncthreads();
+    if (t0 + TS_CHUNK < end) fetch(t0 + TS_CHUNK);  // on its way while this chunk is worked on
+    const int count = min(TS_CHUNK, end - t0);
+    for (int j = 0; j < count; ++j) {
+      const float vc = lv[j][c];
+      float acc = 0.f;
+#pragma unroll
+      for (int a4 = 0; a4 < RPL / 4; ++a4) {
+        const float4 r4 = *reinterpret_cast<const float4*>(&lr[j][i0 + 4 * a4]);
+        const float4 k4 = *reinterpret_cast<const float4*>(&lk[j][i0 + 4 * a4]);
+        const float4 w4 = *reinterpret_cast<const float4*>(&lw[j][i0 + 4 * a4]);
+        const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, ww[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const int a = 4 * a4 + b;
+          const float kv = kk[b] * vc;
+          acc = fmaf(rr[b], fmaf(u[a], kv, s[a]), acc);
+          s[a] = fmaf(ww[b], s[a], kv);
+        }
+      }
+      acc += __shfl_xor(acc, 16, ME_WAVE);
+      acc += __shfl_xor(acc, 32, ME_WAVE);
+      if (p == 0) o[(size_t)(t0 + j) * n + head * D + c] = acc;
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < RPL; ++a) S[(size_t)(i0 + a) * D + c] = s[a];
+}
+
 // A wave per (token, head): o over its root mean square, times the weight, silu(gate) and the scale, into out at column out_col.
 template <typename T>
 __global__ __launch_bounds__(256) void time_finish_kernel(const float* __restrict__ o, const T* __restrict__ gate, const float* __restrict__ w,
@@ -179,10 +290,23 @@ extern "C" int me_time_mix(const void* r, const void* k, const void* v, const vo
   const unsigned scan_blocks = (unsigned)(items * heads * ((d + 15) / 16));
   const long long units = (long long)num_tokens * heads;
   const unsigned fin_blocks = (unsigned)((units + 3) / 4);
+  // steps that bring an item more than a token or two, heads of 32, 64 or 128 elements, rows at multiples of 16 bytes: the kernel that
+  // stages chunks of tokens in LDS
+  const bool chunked = num_tokens >= 4 * items && (d == 32 || d == 64 || d == 128) &&
+                       ((((uintptr_t)r | (uintptr_t)k | (uintptr_t)v | (uintptr_t)decay)) & 15) == 0;
 #define ME_TM_RUN(TT)                                                                                                               \
   do {                                                                                                                              \
     time_decay_kernel<TT><<<num_tokens, 256, 0, stream>>>((const TT*)z, (const TT*)W2, w0, decay, (int)n, rank);                    \
-    if (d <= 32)                                                                                                                    \
+    if (chunked && d == 32)                                                                                                         \
+      time_scan_chunked_kernel<TT, 32><<<items * heads, 128, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, \
+                                                                          state_row, state_slots, item_start, o, heads);           \
+    else if (chunked && d == 64)                                                                                                    \
+      time_scan_chunked_kernel<TT, 64><<<items * heads, 256, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, \
+                                                                          state_row, state_slots, item_start, o, heads);           \
+    else if (chunked && d == 128)                                                                                                   \
+      time_scan_chunked_kernel<TT, 128><<<items * heads, 512, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, \
+                                                                           state_row, state_slots, item_start, o, heads);          \
+    else if (d <= 32)                                                                                                                    \
       time_scan_kernel<TT, 8><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
                                                               state_slots, item_start, o, heads, d);                                \
     else if (d <= 64)                                                                                                               \
