@@ -14,8 +14,10 @@
 // taps]; state float32 [slots, taps - 1, nq + nk + nv]; rotary table float32 [positions, 2, rotary/2] (cosines, then sines).
 #include "common.h"
 
-template <typename T>
-__global__ __launch_bounds__(256) void conv_norm_rope_scatter_kernel(
+// TMAX: the most taps this instance takes (its loops over taps are unrolled to that many, so that all of a thread's loads, of four
+// channels at a time, are on their way together: a step of single tokens waits for memory once, not once per channel and tap).
+template <typename T, int TMAX>
+__global__ __launch_bounds__(1024) void conv_norm_rope_scatter_kernel(
     const T* __restrict__ proj, long long row, int c_q, int c_k, int c_v, const float* __restrict__ conv_w, int taps,
     const float* __restrict__ state, const int* __restrict__ state_slots, const int* __restrict__ item_start,
     const float* __restrict__ q_w, const float* __restrict__ k_w, const float* __restrict__ rope, int rotary,
@@ -31,26 +33,44 @@ __global__ __launch_bounds__(256) void conv_norm_rope_scatter_kernel(
   const float* srow = taps > 1 ? state + (size_t)state_slots[item] * (taps - 1) * C : nullptr;
   auto column = [&](int c) { return c < nq ? c_q + c : (c < nq + nk ? c_k + (c - nq) : c_v + (c - nq - nk)); };
   float sq = 0.f, sk = 0.f;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    const int col = column(c);
-    float y;
-    if (taps > 0) {
-      y = 0.f;
-      for (int j = 0; j < taps; ++j) {
-        const int back = taps - 1 - j;
-        if (pos - back < 0) continue;  // before the sequence's first token: zeros
-        const int from = t - back;
-        const float u = from >= first ? to_float(proj[(size_t)from * row + col])
-                                      : to_float(from_float<T>(srow[(size_t)(taps - 1 - (first - from)) * C + c]));
-        y = fmaf(conv_w[(size_t)c * taps + j], u, y);
+  constexpr int U = 4;  // channels a thread has in flight
+  for (int c0 = threadIdx.x; c0 < C; c0 += U * blockDim.x) {
+    float u[U][TMAX > 0 ? TMAX : 1], w[U][TMAX > 0 ? TMAX : 1], plain[U];
+#pragma unroll
+    for (int a = 0; a < U; ++a) {
+      const int c = c0 + a * blockDim.x;
+      const bool there = c < C;
+      const int col = column(there ? c : 0);
+      plain[a] = 0.f;
+      if (TMAX == 0) {
+        if (there) plain[a] = to_float(proj[(size_t)t * row + col]);
+        continue;
       }
-      y = to_float(from_float<T>(y));  // (the convolution's result in the activations' type, as a product's would be)
-    } else {
-      y = to_float(proj[(size_t)t * row + col]);
+#pragma unroll
+      for (int j = 0; j < TMAX; ++j) {
+        const int back = taps - 1 - j, from = t - back;
+        u[a][j] = w[a][j] = 0.f;
+        if (there && j < taps && pos - back >= 0) {  // (before the sequence's first token: zeros)
+          u[a][j] = from >= first ? to_float(proj[(size_t)from * row + col]) : srow[(size_t)(taps - 1 - (first - from)) * C + c];
+          w[a][j] = conv_w[(size_t)c * taps + j];
+        }
+      }
     }
-    vals[c] = y;
-    if (c < nq) sq = fmaf(y, y, sq);
-    else if (c < nq + nk) sk = fmaf(y, y, sk);
+#pragma unroll
+    for (int a = 0; a < U; ++a) {
+      const int c = c0 + a * blockDim.x;
+      if (c >= C) continue;
+      float y = plain[a];
+      if (TMAX > 0) {
+        y = 0.f;
+#pragma unroll
+        for (int j = 0; j < TMAX; ++j) y = fmaf(w[a][j], u[a][j], y);  // (taps beyond the layer's, or before the sequence: zeros)
+        y = to_float(from_float<T>(y));  // (the convolution's result in the activations' type, as a product's would be)
+      }
+      vals[c] = y;
+      if (c < nq) sq = fmaf(y, y, sq);
+      else if (c < nq + nk) sk = fmaf(y, y, sk);
+    }
   }
   const float rq = rsqrtf(block_sum(sq, red) / (float)nq + eps);
   const float rk = rsqrtf(block_sum(sk, red) / (float)nk + eps);
@@ -129,20 +149,35 @@ extern "C" int me_conv_norm_rope_scatter(const void* proj, long long row, int c_
   const size_t lds = (size_t)C * sizeof(float);
   if (lds > 60 * 1024) return me_fail("me_conv_norm_rope_scatter: rows of %lld elements do not fit a block's memory", C);
   if (!item_start) return me_fail("me_conv_norm_rope_scatter: no item boundaries");
+  // few tokens (decode steps): a block of 1,024 threads, so that a token's channels are fetched in one or two rounds
+  const int threads = num_tokens <= 256 && C > 1024 ? 1024 : 256;
+#define ME_CS_LAUNCH(TT, TM)                                                                                                          \
+  conv_norm_rope_scatter_kernel<TT, TM><<<num_tokens, threads, lds, stream>>>(                                                          \
+      (const TT*)proj, row, c_q, c_k, c_v, conv_w, taps, state, state_slots, item_start, q_w, k_w, rope, rotary, positions, token_item, \
+      block_table, table_width, (TT*)q_out, (TT*)k_cache, (TT*)v_cache, nh, nkv, d, dv, bs, eps)
+#define ME_CS_RUN(TT)                 \
+  do {                                \
+    if (taps == 0)                    \
+      ME_CS_LAUNCH(TT, 0);            \
+    else if (taps <= 4)               \
+      ME_CS_LAUNCH(TT, 4);            \
+    else if (taps <= 8)               \
+      ME_CS_LAUNCH(TT, 8);            \
+    else                              \
+      ME_CS_LAUNCH(TT, CS_MAX_TAPS);  \
+  } while (0)
   if (dtype == ME_F32) {
-    conv_norm_rope_scatter_kernel<float><<<num_tokens, 256, lds, stream>>>(
-        (const float*)proj, row, c_q, c_k, c_v, conv_w, taps, state, state_slots, item_start, q_w, k_w, rope, rotary, positions, token_item,
-        block_table, table_width, (float*)q_out, (float*)k_cache, (float*)v_cache, nh, nkv, d, dv, bs, eps);
+    ME_CS_RUN(float);
     if (taps > 1)
       conv_state_keep_kernel<float><<<items, 256, 0, stream>>>((const float*)proj, row, c_q, c_k, c_v, state, state_slots, item_start, taps,
                                                                (int)nq, (int)nk, (int)nv);
   } else {
-    conv_norm_rope_scatter_kernel<bf16_t><<<num_tokens, 256, lds, stream>>>(
-        (const bf16_t*)proj, row, c_q, c_k, c_v, conv_w, taps, state, state_slots, item_start, q_w, k_w, rope, rotary, positions,
-        token_item, block_table, table_width, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, dv, bs, eps);
+    ME_CS_RUN(bf16_t);
     if (taps > 1)
       conv_state_keep_kernel<bf16_t><<<items, 256, 0, stream>>>((const bf16_t*)proj, row, c_q, c_k, c_v, state, state_slots, item_start,
                                                                 taps, (int)nq, (int)nk, (int)nv);
   }
+#undef ME_CS_RUN
+#undef ME_CS_LAUNCH
   return me_check_launch("me_conv_norm_rope_scatter");
 }

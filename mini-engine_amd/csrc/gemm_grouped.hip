@@ -23,12 +23,14 @@ typedef __attribute__((address_space(3))) void* gg_lds_ptr;
 namespace {
 constexpr int GGK = 64;  // k per LDS tile; also the LDS row length in elements
 
-template <int BM, int BN, int WM, int WN, bool GATED>
+// MODE 0: the down product; 1: gate and up rows; 2: up rows alone (experts without a gate: act(x_e . Wu_e^T) -> acts).
+template <int BM, int BN, int WM, int WN, int MODE>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_grouped_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                                      const int* __restrict__ plan, const int* __restrict__ sorted,
                                                                      const float* __restrict__ wts, bf16_t* __restrict__ acts,
                                                                      float* __restrict__ parts, int num_tokens, int N, int K,
                                                                      int top, int n_tiles, int gate, float limit) {
+  constexpr bool GATED = MODE == 1, GATHER = MODE != 0;
   constexpr int THREADS = WM * WN * 64;
   constexpr int WMR = BM / WM, WNR = BN / WN;
   constexpr int FM = WMR / 16, FN = WNR / 16;
@@ -54,7 +56,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_grouped_kernel(const bf16_t
   for (int i = 0; i < NX; ++i) {
     const int tr = (tid + i * THREADS) >> 3;
     const int at = begin + min(tr, rows - 1);
-    const size_t row = GATED ? (size_t)(sorted[at] / top) : (size_t)at;
+    const size_t row = GATHER ? (size_t)(sorted[at] / top) : (size_t)at;
     px[i] = X + row * K + (((tid & 7) ^ ((tr >> 1) & 7)) * 8);
   }
   const int w_rows = GATED ? 2 * N : N;
@@ -135,6 +137,15 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_grouped_kernel(const bf16_t
             if (n + i < N) p[i] = from_float<bf16_t>(v[i]);
         }
       }
+    } else if constexpr (GATHER) {
+#pragma unroll
+      for (int a = 0; a < FN; ++a) {
+        const int n = n0 + wn * WNR + a * 16 + 4 * g;
+        bf16_t* p = acts + (size_t)(begin + m) * N + n;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) p[i] = from_float<bf16_t>(ungated_act(acc[a][b][i], gate));
+      }
     } else {
       const int pair = sorted[begin + m];
       const float wgt = wts[pair];
@@ -154,13 +165,13 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_grouped_kernel(const bf16_t
   }
 }
 
-template <bool GATED>
+template <int MODE>
 int launch_grouped(const bf16_t* X, const bf16_t* W, const int* plan, const int* sorted, const float* wts, bf16_t* acts, float* parts,
                    int num_tokens, int N, int K, int top, int max_tiles, int gate, float limit, hipStream_t stream) {
   constexpr int BM = 128, BN = 128, WM = 4, WN = 2;
-  constexpr int COLS = GATED ? BN / 2 : BN;
+  constexpr int COLS = MODE == 1 ? BN / 2 : BN;
   constexpr size_t LDS = (size_t)2 * (BM + BN) * GGK * sizeof(bf16_t);
-  auto kernel = gemm_grouped_kernel<BM, BN, WM, WN, GATED>;
+  auto kernel = gemm_grouped_kernel<BM, BN, WM, WN, MODE>;
   static bool raised = false;
   if (!raised) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS) != hipSuccess)
@@ -187,9 +198,12 @@ extern "C" int me_gemm_grouped_bf16(const void* X, const void* W, const int* pla
   if (num_tokens <= 0 || max_tiles <= 0) return 0;
   if (K <= 0 || K % GGK) return me_fail("me_gemm_grouped: K=%d must be a positive multiple of %d", K, GGK);
   if (((uintptr_t)X | (uintptr_t)W) & 15) return me_fail("me_gemm_grouped: operands must be 16-byte aligned");
+  if (act_is_ungated(gated))  // an activation without a gate: W [E, N, K], acts [P, N] = act(x_e . W_e^T), x rows gathered by token
+    return launch_grouped<2>((const bf16_t*)X, (const bf16_t*)W, plan, sorted, wts, (bf16_t*)acts, nullptr, num_tokens, N, K, top,
+                             max_tiles, gated, limit, stream);
   if (gated)
-    return launch_grouped<true>((const bf16_t*)X, (const bf16_t*)W, plan, sorted, wts, (bf16_t*)acts, nullptr, num_tokens, N, K, top,
+    return launch_grouped<1>((const bf16_t*)X, (const bf16_t*)W, plan, sorted, wts, (bf16_t*)acts, nullptr, num_tokens, N, K, top,
                                 max_tiles, gated, limit, stream);
-  return launch_grouped<false>((const bf16_t*)X, (const bf16_t*)W, plan, sorted, wts, nullptr, parts, num_tokens, N, K, top, max_tiles, 0,
+  return launch_grouped<0>((const bf16_t*)X, (const bf16_t*)W, plan, sorted, wts, nullptr, parts, num_tokens, N, K, top, max_tiles, 0,
                                0.f, stream);
 }

@@ -457,12 +457,13 @@ extern "C" int me_routed_ff_routed(const void* h, const float* Wr, const void* W
                                                                  parts, num_tokens, hidden, ff, top, act, limit);
       return finish();
     }
-    if (!ungated && P >= 96ll * E && hidden % 64 == 0 && ff % 64 == 0) {
+    if (P >= 96ll * E && hidden % 64 == 0 && ff % 64 == 0) {
       // prompts: tiles of 128 pairs through the product that stages both operands in LDS (gemm_grouped.hip)
       const int rows128 = me_gemm_grouped_tile_rows(), tiles128 = (int)((P + rows128 - 1) / rows128) + E;
       routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, rows128, plan, sorted, n_identity);
       if (me_gemm_grouped_bf16(h, W_gu, plan, sorted, wts, acts, nullptr, num_tokens, ff, hidden, top, tiles128, act, limit, stream)) return 1;
-      return me_gemm_grouped_bf16(acts, W_down, plan, sorted, wts, nullptr, parts, num_tokens, hidden, ff, top, tiles128, 0, 0.f, stream);
+      if (me_gemm_grouped_bf16(acts, W_down, plan, sorted, wts, nullptr, parts, num_tokens, hidden, ff, top, tiles128, 0, 0.f, stream)) return 1;
+      return finish();
     }
     routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, wide ? 64 : 16, plan, sorted, n_identity);
     if (wide) {

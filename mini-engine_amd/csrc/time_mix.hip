@@ -70,22 +70,7 @@ extern "C" int me_time_shift(const void* h, float* state, long long state_row, l
   return me_check_launch("me_time_shift");
 }
 
-// decay[t, c] = exp(-exp(sum_j W2[c, j] tanh(z[t, j]) + w0[c])). Grid (tokens), a thread a channel in turns.
 #define TM_MAX_RANK 1024
-template <typename T>
-__global__ __launch_bounds__(256) void time_decay_kernel(const T* __restrict__ z, const T* __restrict__ W2, const float* __restrict__ w0,
-                                                         float* __restrict__ decay, int n, int rank) {
-  __shared__ float th[TM_MAX_RANK];
-  const int t = blockIdx.x;
-  for (int j = threadIdx.x; j < rank; j += blockDim.x) th[j] = tanhf(to_float(z[(size_t)t * rank + j]));
-  __syncthreads();
-  for (int c = threadIdx.x; c < n; c += blockDim.x) {
-    const T* wr = W2 + (size_t)c * rank;
-    float s = 0.f;
-    for (int j = 0; j < rank; ++j) s = fmaf(to_float(wr[j]), th[j], s);
-    decay[(size_t)t * n + c] = expf(-expf(s + w0[c]));
-  }
-}
 
 // A wave per (item, head, group of 16 value channels); RPL: rows of S a lane holds (d <= 4 * RPL).
 template <typename T, int RPL>
@@ -174,6 +159,50 @@ struct TsVec<float> {
     *reinterpret_cast<float4*>(dst + 4) = b;
   }
 };
+
+// decay[t, c] = exp(-exp(sum_j W2[c, j] tanh(z[t, j]) + w0[c])). Grid (runs of TD_TOKENS tokens, runs of 256 channels), a thread a
+// channel: it walks its row of W2 eight elements a load and meets every token of the run with each piece, so that a row is fetched
+// once for the run's tokens. The sum over j runs in ascending j for every token, whatever else the step holds.
+#define TD_TOKENS 8
+template <typename T>
+__global__ __launch_bounds__(256) void time_decay_kernel(const T* __restrict__ z, const T* __restrict__ W2, const float* __restrict__ w0,
+                                                         float* __restrict__ decay, int num_tokens, int n, int rank) {
+  extern __shared__ float th[];  // [TD_TOKENS][rank]
+  const int t0 = blockIdx.x * TD_TOKENS, count = min(TD_TOKENS, num_tokens - t0);
+  for (int i = threadIdx.x; i < count * rank; i += blockDim.x) th[i] = tanhf(to_float(z[(size_t)t0 * rank + i]));
+  __syncthreads();
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= n) return;
+  const T* wr = W2 + (size_t)c * rank;
+  float sum[TD_TOKENS];
+#pragma unroll
+  for (int k = 0; k < TD_TOKENS; ++k) sum[k] = 0.f;
+  const bool vec = rank % 8 == 0 && (((uintptr_t)W2) & 15) == 0;
+  int j = 0;
+  if (vec)
+    for (; j + 8 <= rank; j += 8) {
+      TsVec<T> piece;
+      piece.load(wr + j);
+      __attribute__((aligned(16))) float w8[8];
+      piece.store(w8);
+#pragma unroll
+      for (int k = 0; k < TD_TOKENS; ++k)
+        if (k < count) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) sum[k] = fmaf(w8[i], th[k * rank + j + i], sum[k]);
+        }
+    }
+  for (; j < rank; ++j) {
+    const float w = to_float(wr[j]);
+#pragma unroll
+    for (int k = 0; k < TD_TOKENS; ++k)
+      if (k < count) sum[k] = fmaf(w, th[k * rank + j], sum[k]);
+  }
+  const float bias = w0[c];
+#pragma unroll
+  for (int k = 0; k < TD_TOKENS; ++k)
+    if (k < count) decay[(size_t)(t0 + k) * n + c] = expf(-expf(sum[k] + bias));
+}
 
 template <typename T, int D>
 __global__ __launch_bounds__(4 * D) void time_scan_chunked_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v,
@@ -296,7 +325,9 @@ extern "C" int me_time_mix(const void* r, const void* k, const void* v, const vo
                        ((((uintptr_t)r | (uintptr_t)k | (uintptr_t)v | (uintptr_t)decay)) & 15) == 0;
 #define ME_TM_RUN(TT)                                                                                                               \
   do {                                                                                                                              \
-    time_decay_kernel<TT><<<num_tokens, 256, 0, stream>>>((const TT*)z, (const TT*)W2, w0, decay, (int)n, rank);                    \
+    time_decay_kernel<TT><<<dim3((num_tokens + TD_TOKENS - 1) / TD_TOKENS, (unsigned)((n + 255) / 256)), 256,                       \
+                            (size_t)TD_TOKENS * rank * sizeof(float), stream>>>((const TT*)z, (const TT*)W2, w0, decay, num_tokens,  \
+                                                                                (int)n, rank);                                      \
     if (chunked && d == 32)                                                                                                         \
       time_scan_chunked_kernel<TT, 32><<<items * heads, 128, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, \
                                                                           state_row, state_slots, item_start, o, heads);           \
