@@ -395,7 +395,7 @@ class StepProgram:
                   activation_limit: float = 0.0, scoring: str = "softmax_picked", num_groups: int = 1, keep_groups: int = 1,
                   route_scale: float = 1.0, shared_gate_up: torch.Tensor | None = None, shared_down: torch.Tensor | None = None,
                   shared_limit: float = 0.0, identity_experts: int = 0, correction: torch.Tensor | None = None,
-                  shared_gated: bool = True) -> None:
+                  shared_gated: bool = True, gated: bool = True) -> None:
         """A feed-forward of routed experts on the value ``x`` as the part's result. ``router`` float32 ``[experts, hidden]``;
         ``gate_up`` ``[experts, 2 ff, hidden]`` (an expert's gate rows, then its up rows) and ``down`` ``[experts, hidden, ff]``
         in the compute dtype. ``scoring``, ``num_groups``, ``keep_groups``, ``route_scale``: how the picks are bounded and weighted
@@ -404,11 +404,13 @@ class StepProgram:
         product with which, through a sigmoid, multiplies that expert's result."""
         from ..ops.kernels import UNGATED_ACTIVATIONS, gate_code
 
-        # An activation of UNGATED_ACTIVATIONS: the experts have no gate, ``gate_up`` is ``[experts, ff, hidden]`` (up rows alone) and
+        # ``gated`` false (an activation of UNGATED_ACTIVATIONS): the experts have no gate, ``gate_up`` is ``[experts, ff, hidden]`` (up rows alone) and
         # ``shared_gate_up`` ``[ff_s, hidden]``. ``identity_experts``: that many router outputs behind the experts' stand for identity
         # experts (the token's input itself, times the weight); ``correction`` float32 ``[experts + identity_experts]`` is added to the
         # scores for the choice alone (scoring "softmax_all"). ``shared_gated`` false: nothing multiplies the shared expert's result.
-        ungated = activation in UNGATED_ACTIVATIONS
+        ungated = not gated
+        if ungated and activation not in UNGATED_ACTIVATIONS:
+            raise ValueError(f"experts without a gate know the activations {sorted(UNGATED_ACTIVATIONS)}, got {activation!r}")
         experts, two_ff, hidden = gate_up.shape
         if ungated:
             two_ff *= 2

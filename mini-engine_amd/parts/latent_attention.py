@@ -57,15 +57,13 @@ class LatentAttention(Mixer):
     # ---- weights
     def weight_wants(self, prefix: str) -> dict[str, TensorWant]:
         s, n = self.spec, self._n
-        wants = {
-            f"{prefix}.{n['q']}": TensorWant((self.nh * (self.d + self.r), s.hidden_size)),
-            f"{prefix}.{n['uk']}": TensorWant((self.nh * self.d, self.rank)),
-            f"{prefix}.{n['uv']}": TensorWant((self.nh * self.dv, self.rank)),
-            f"{prefix}.{n['o']}": TensorWant((s.hidden_size, self.nh * self.dv)),
-        }
-        if self.cache_from is None:
+        wants = {f"{prefix}.{n['q']}": TensorWant((self.nh * (self.d + self.r), s.hidden_size))}
+        if self.cache_from is None:  # (a layer that reads another layer's pages has no latent projection of its own)
             wants[f"{prefix}.{n['dkv']}"] = TensorWant((self.rank + self.r, s.hidden_size))
             wants[f"{prefix}.{n['dkv_norm']}"] = TensorWant((self.rank,), "vector")
+        wants[f"{prefix}.{n['uk']}"] = TensorWant((self.nh * self.d, self.rank))
+        wants[f"{prefix}.{n['uv']}"] = TensorWant((self.nh * self.dv, self.rank))
+        wants[f"{prefix}.{n['o']}"] = TensorWant((s.hidden_size, self.nh * self.dv))
         if s.sink:
             wants[f"{prefix}.{n['sink']}"] = TensorWant((self.nh,), "vector")
         if s.output_gate:

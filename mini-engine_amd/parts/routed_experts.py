@@ -108,7 +108,7 @@ class RoutedExperts(FeedForward):
                           keep_groups=self.keep, route_scale=float(getattr(s, "route_scale", 1.0)),
                           shared_gate_up=self.w_shared_gate_up, shared_down=self.w_shared_down,
                           shared_limit=float(getattr(s, "shared_limit", 0.0)), identity_experts=self.identity, correction=self.correction,
-                          shared_gated=self.shared_gated)
+                          shared_gated=self.shared_gated, gated=self.gated)
 
 
 FEED_FORWARDS.register("routed_experts", RoutedExperts)

@@ -15,7 +15,7 @@ import trace_helpers as th
 
 pytestmark = pytest.mark.gpu
 
-SEEDS = {"A": 1, "B": 4, "C": 1, "D": 1}  # (seeds whose routers decide nothing by a hair for the first dozens of tokens)
+SEEDS = {"A": 3, "B": 4, "C": 1, "D": 1}  # (seeds whose routers decide nothing by a hair for the first dozens of tokens)
 LENGTHS = {"long": 150, "mid": 61, "short": 5, "one": 1, "pair": 2, "other": 37}
 
 
