@@ -8,9 +8,11 @@
 //   shift    for every token the five blends (r, k, v, gate, decay) in the activations' type; h' of an item's first token is the
 //            item's state row (zeros at position 0). A second launch keeps the item's last input as the next h'.
 //   decay    w = exp(-exp(W_2 tanh(z) + w_0)) in float32 for all tokens, z the decay's inner projection.
-//   scan     a wave per (item, head, 16 value channels): lane (p, c) holds a quarter of the rows of column c of S and walks the
-//            item's tokens; the quarters' sums meet through two exchanges. Sums run in an order that the head's size alone
-//            fixes, so a token's result does not depend on how the sequence was cut or on what else the step holds.
+//   scan     a wave per (item, head, 4 value channels): a row of 16 lanes a column of S, each lane d / 16 of the column's rows in
+//            registers; the wave walks the item's tokens, and a column's sum over its row of lanes is four data-parallel moves.
+//            Sums run in an order that the head's size alone fixes (a lane's rows in ascending order, then the row of lanes
+//            pairwise), in both forms of the kernel: a token's result is the same bits however the sequence was cut and whatever
+//            else the step holds.
 //   finish   every head's o over its root mean square, times a weight, times silu(gate), times the caller's scale.
 //
 // State row of a slot: [heads, d (key), d (value)] float32, then the `width` elements of h'.
@@ -72,16 +74,30 @@ extern "C" int me_time_shift(const void* h, float* state, long long state_row, l
 
 #define TM_MAX_RANK 1024
 
-// A wave per (item, head, group of 16 value channels); RPL: rows of S a lane holds (d <= 4 * RPL).
+// A column's sum over its row of 16 lanes (the lanes of a wave whose numbers differ in their low four bits), in every lane of the
+// row, by four data-parallel moves (no LDS): a rotation by 8, one by 4, then the two exchanges inside a group of four add the same
+// pairs in every lane, so all lanes hold the same bits.
+__device__ __forceinline__ float row16_sum(float x) {
+#define TM_DPP_ADD(CTRL) x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false))
+  TM_DPP_ADD(0x128);  // row_ror:8
+  TM_DPP_ADD(0x124);  // row_ror:4
+  TM_DPP_ADD(0x4e);   // quad_perm:[2,3,0,1]
+  TM_DPP_ADD(0xb1);   // quad_perm:[1,0,3,2]
+#undef TM_DPP_ADD
+  return x;
+}
+
+// A wave per (item, head, group of 4 value channels); RPL: rows of S a lane holds (d <= 16 * RPL). Lane l: column 4 * group + l / 16,
+// rows (l % 16) * per .. + per - 1 with per = ceil(d / 16).
 template <typename T, int RPL>
 __global__ __launch_bounds__(64) void time_scan_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v,
                                                        const float* __restrict__ decay, const float* __restrict__ bonus,
                                                        float* __restrict__ state, long long state_row, const int* __restrict__ state_slots,
                                                        const int* __restrict__ item_start, float* __restrict__ o, int heads, int d) {
-  const int groups = (d + 15) / 16;
+  const int groups = (d + 3) / 4;
   const int item = blockIdx.x / (heads * groups), head = (blockIdx.x / groups) % heads, grp = blockIdx.x % groups;
-  const int lane = threadIdx.x, p = lane >> 4, c = grp * 16 + (lane & 15);
-  const int per = (d + 3) / 4, i0 = p * per;
+  const int lane = threadIdx.x, rp = lane & 15, c = grp * 4 + (lane >> 4);
+  const int per = (d + 15) / 16, i0 = rp * per;
   const int first = item_start[item], end = item_start[item + 1];
   const bool col = c < d;
   const int n = heads * d;
@@ -113,9 +129,8 @@ __global__ __launch_bounds__(64) void time_scan_kernel(const T* __restrict__ r, 
       acc = fmaf(rr[a], fmaf(u[a], kv, s[a]), acc);
       s[a] = fmaf(ww[a], s[a], kv);
     }
-    acc += __shfl_xor(acc, 16, ME_WAVE);
-    acc += __shfl_xor(acc, 32, ME_WAVE);
-    if (p == 0 && col) o[at + c] = acc;
+    acc = row16_sum(acc);
+    if (rp == 0 && col) o[at + c] = acc;
   }
 #pragma unroll
   for (int a = 0; a < RPL; ++a) {
@@ -124,11 +139,11 @@ __global__ __launch_bounds__(64) void time_scan_kernel(const T* __restrict__ r, 
   }
 }
 
-// The scan for heads of D = 32, 64 or 128 elements, a block per (item, head) and a wave per 16 value channels of it. The block walks the
-// item's tokens in chunks of TS_CHUNK: all threads fetch a chunk's r, k, v and decays together (16 bytes a load, every load of the chunk
-// in flight at once, and the next chunk's asked for before this one is worked on) and lay them out in LDS as float32; then every wave
-// walks the chunk's tokens out of LDS. The sums are those of time_scan_kernel, in its order: a token's result is the same bits
-// whichever of the two kernels serves it.
+// The scan for heads of D = 32, 64 or 128 elements, a block of four waves per (item, head, 16 value channels), a wave per 4 of them. The
+// block walks the item's tokens in chunks of TS_CHUNK (half as many for heads of 128): all threads fetch a chunk's r, k and decays (the head's whole rows) and the v of
+// the block's channels together (16 bytes a load, every load of the chunk in flight at once, and the next chunk's asked for before
+// this one is worked on) and lay them out in LDS as float32; then every wave walks the chunk's tokens out of LDS. The sums are those
+// of time_scan_kernel, in its order: a token's result is the same bits whichever of the two kernels serves it.
 #define TS_CHUNK 32
 template <typename T>
 struct TsVec;  // eight consecutive elements of a row
@@ -205,16 +220,19 @@ __global__ __launch_bounds__(256) void time_decay_kernel(const T* __restrict__ z
 }
 
 template <typename T, int D>
-__global__ __launch_bounds__(4 * D) void time_scan_chunked_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v,
-                                                                 const float* __restrict__ decay, const float* __restrict__ bonus,
-                                                                 float* __restrict__ state, long long state_row,
-                                                                 const int* __restrict__ state_slots, const int* __restrict__ item_start,
-                                                                 float* __restrict__ o, int heads) {
-  constexpr int RPL = D / 4, VPR = D / 8;  // rows of S a lane holds; vectors of eight elements a row
-  __shared__ __attribute__((aligned(16))) float lr[TS_CHUNK][D], lk[TS_CHUNK][D], lv[TS_CHUNK][D], lw[TS_CHUNK][D];
-  const int item = blockIdx.x / heads, head = blockIdx.x % heads;
+__global__ __launch_bounds__(256) void time_scan_chunked_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v,
+                                                                const float* __restrict__ decay, const float* __restrict__ bonus,
+                                                                float* __restrict__ state, long long state_row,
+                                                                const int* __restrict__ state_slots, const int* __restrict__ item_start,
+                                                                float* __restrict__ o, int heads) {
+  constexpr int RPL = D / 16, VPR = D / 8;       // rows of S a lane holds; vectors of eight elements a row
+  constexpr int CH = D > 64 ? TS_CHUNK / 2 : TS_CHUNK;  // tokens a chunk: a thread fetches one vector of each array
+  constexpr int NV = (CH * VPR + 255) / 256;  // vectors of a chunk's r (k, decays) a thread fetches
+  constexpr int PARTS = D / 16;                  // blocks a head
+  __shared__ __attribute__((aligned(16))) float lr[CH][D], lk[CH][D], lw[CH][D], lv[CH][16];
+  const int item = blockIdx.x / (heads * PARTS), head = (blockIdx.x / PARTS) % heads, part = blockIdx.x % PARTS;
   const int tid = threadIdx.x, wave = tid / ME_WAVE, lane = tid & (ME_WAVE - 1);
-  const int p = lane >> 4, c = wave * 16 + (lane & 15), i0 = p * RPL;
+  const int rp = lane & 15, cl = wave * 4 + (lane >> 4), c = part * 16 + cl, i0 = rp * RPL;
   const int first = item_start[item], end = item_start[item + 1];
   const int n = heads * D;
   float* S = state + (size_t)state_slots[item] * state_row + (size_t)head * D * D;
@@ -224,56 +242,81 @@ __global__ __launch_bounds__(4 * D) void time_scan_chunked_kernel(const T* __res
     s[a] = S[(size_t)(i0 + a) * D + c];
     u[a] = bonus[head * D + i0 + a];
   }
-  // this thread's vector of a chunk: token tid / VPR of the chunk, elements 8 (tid % VPR) .. + 7 of the head's row
-  const int vt = tid / VPR, ve = 8 * (tid % VPR);
-  TsVec<T> fr, fk, fv;
-  float4 fw0, fw1;
+  TsVec<T> fr[NV], fk[NV], fv;
+  float4 fw0[NV], fw1[NV];
   auto fetch = [&](int t0) {
-    const int t = t0 + vt;
-    if (t < end) {
-      const size_t at = (size_t)t * n + head * D + ve;
-      fr.load(r + at);
-      fk.load(k + at);
-      fv.load(v + at);
-      fw0 = *reinterpret_cast<const float4*>(decay + at);
-      fw1 = *reinterpret_cast<const float4*>(decay + at + 4);
-    } else {
-      fr.zero(), fk.zero(), fv.zero();
-      fw0 = fw1 = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+      const int vi = tid + 256 * q, t = t0 + vi / VPR, ve = 8 * (vi % VPR);
+      if (vi < CH * VPR && t < end) {
+        const size_t at = (size_t)t * n + head * D + ve;
+        fr[q].load(r + at);
+        fk[q].load(k + at);
+        fw0[q] = *reinterpret_cast<const float4*>(decay + at);
+        fw1[q] = *reinterpret_cast<const float4*>(decay + at + 4);
+      } else {
+        fr[q].zero(), fk[q].zero();
+        fw0[q] = fw1[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+      }
     }
+    fv.zero();
+    if (tid < CH * 2 && t0 + tid / 2 < end)  // the block's 16 value channels: two vectors a token
+      fv.load(v + (size_t)(t0 + tid / 2) * n + head * D + part * 16 + 8 * (tid % 2));
   };
   if (first < end) fetch(first);
-  for (int t0 = first; t0 < end; t0 += TS_CHUNK) {
+  for (int t0 = first; t0 < end; t0 += CH) {
     __syncthreads();  // the chunk before is worked off
-    fr.store(&lr[vt][ve]);
-    fk.store(&lk[vt][ve]);
-    fv.store(&lv[vt][ve]);
-    *reinterpret_cast<float4*>(&lw[vt][ve]) = fw0;
-    *reinterpret_cast<float4*>(&lw[vt][ve + 4]) = fw1;
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+      const int vi = tid + 256 * q, vt = vi / VPR, ve = 8 * (vi % VPR);
+      if (vi < CH * VPR) {
+        fr[q].store(&lr[vt][ve]);
+        fk[q].store(&lk[vt][ve]);
+        *reinterpret_cast<float4*>(&lw[vt][ve]) = fw0[q];
+        *reinterpret_cast<float4*>(&lw[vt][ve + 4]) = fw1[q];
+      }
+    }
+    if (tid < CH * 2) fv.store(&lv[tid / 2][8 * (tid % 2)]);
     __syncthreads();
-    if (t0 + TS_CHUNK < end) fetch(t0 + TS_CHUNK);  // on its way while this chunk is worked on
-    const int count = min(TS_CHUNK, end - t0);
-    for (int j = 0; j < count; ++j) {
-      const float vc = lv[j][c];
+    if (t0 + CH < end) fetch(t0 + CH);  // on its way while this chunk is worked on
+    const int count = min(CH, end - t0);
+    auto token = [&](int j) {
+      const float vc = lv[j][cl];
+      float rr[RPL], kk[RPL], ww[RPL];
+      if constexpr (RPL % 4 == 0) {
+#pragma unroll
+        for (int a4 = 0; a4 < RPL / 4; ++a4) {
+          const float4 r4 = *reinterpret_cast<const float4*>(&lr[j][i0 + 4 * a4]);
+          const float4 k4 = *reinterpret_cast<const float4*>(&lk[j][i0 + 4 * a4]);
+          const float4 w4 = *reinterpret_cast<const float4*>(&lw[j][i0 + 4 * a4]);
+          rr[4 * a4] = r4.x, rr[4 * a4 + 1] = r4.y, rr[4 * a4 + 2] = r4.z, rr[4 * a4 + 3] = r4.w;
+          kk[4 * a4] = k4.x, kk[4 * a4 + 1] = k4.y, kk[4 * a4 + 2] = k4.z, kk[4 * a4 + 3] = k4.w;
+          ww[4 * a4] = w4.x, ww[4 * a4 + 1] = w4.y, ww[4 * a4 + 2] = w4.z, ww[4 * a4 + 3] = w4.w;
+        }
+      } else {
+#pragma unroll
+        for (int a = 0; a < RPL; ++a) rr[a] = lr[j][i0 + a], kk[a] = lk[j][i0 + a], ww[a] = lw[j][i0 + a];
+      }
       float acc = 0.f;
 #pragma unroll
-      for (int a4 = 0; a4 < RPL / 4; ++a4) {
-        const float4 r4 = *reinterpret_cast<const float4*>(&lr[j][i0 + 4 * a4]);
-        const float4 k4 = *reinterpret_cast<const float4*>(&lk[j][i0 + 4 * a4]);
-        const float4 w4 = *reinterpret_cast<const float4*>(&lw[j][i0 + 4 * a4]);
-        const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, ww[4] = {w4.x, w4.y, w4.z, w4.w};
-#pragma unroll
-        for (int b = 0; b < 4; ++b) {
-          const int a = 4 * a4 + b;
-          const float kv = kk[b] * vc;
-          acc = fmaf(rr[b], fmaf(u[a], kv, s[a]), acc);
-          s[a] = fmaf(ww[b], s[a], kv);
-        }
+      for (int a = 0; a < RPL; ++a) {
+        const float kv = kk[a] * vc;
+        acc = fmaf(rr[a], fmaf(u[a], kv, s[a]), acc);
+        s[a] = fmaf(ww[a], s[a], kv);
       }
-      acc += __shfl_xor(acc, 16, ME_WAVE);
-      acc += __shfl_xor(acc, 32, ME_WAVE);
-      if (p == 0) o[(size_t)(t0 + j) * n + head * D + c] = acc;
+      acc = row16_sum(acc);
+      if (rp == 0) o[(size_t)(t0 + j) * n + head * D + c] = acc;
+    };
+    // four tokens a turn without a branch between them: a token's sum over the row of lanes and its store run under the next tokens'
+    // multiply-adds (only the state's way from token to token, one multiply-add a row, is in order)
+    int j = 0;
+    for (; j + 4 <= count; j += 4) {
+      token(j);
+      token(j + 1);
+      token(j + 2);
+      token(j + 3);
     }
+    for (; j < count; ++j) token(j);
   }
 #pragma unroll
   for (int a = 0; a < RPL; ++a) S[(size_t)(i0 + a) * D + c] = s[a];
@@ -316,7 +359,7 @@ extern "C" int me_time_mix(const void* r, const void* k, const void* v, const vo
   if ((long long)heads * d * d > state_row) return me_fail("me_time_mix: state rows of %lld elements", state_row);
   float* decay = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
   float* o = decay + (size_t)num_tokens * n;
-  const unsigned scan_blocks = (unsigned)(items * heads * ((d + 15) / 16));
+  const unsigned scan_blocks = (unsigned)(items * heads * ((d + 3) / 4));
   const long long units = (long long)num_tokens * heads;
   const unsigned fin_blocks = (unsigned)((units + 3) / 4);
   // steps that bring an item more than a token or two, heads of 32, 64 or 128 elements, rows at multiples of 16 bytes: the kernel that
@@ -329,25 +372,25 @@ extern "C" int me_time_mix(const void* r, const void* k, const void* v, const vo
                             (size_t)TD_TOKENS * rank * sizeof(float), stream>>>((const TT*)z, (const TT*)W2, w0, decay, num_tokens,  \
                                                                                 (int)n, rank);                                      \
     if (chunked && d == 32)                                                                                                         \
-      time_scan_chunked_kernel<TT, 32><<<items * heads, 128, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, \
+      time_scan_chunked_kernel<TT, 32><<<items * heads * 2, 256, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, \
                                                                           state_row, state_slots, item_start, o, heads);           \
     else if (chunked && d == 64)                                                                                                    \
-      time_scan_chunked_kernel<TT, 64><<<items * heads, 256, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, \
+      time_scan_chunked_kernel<TT, 64><<<items * heads * 4, 256, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, \
                                                                           state_row, state_slots, item_start, o, heads);           \
     else if (chunked && d == 128)                                                                                                   \
-      time_scan_chunked_kernel<TT, 128><<<items * heads, 512, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, \
+      time_scan_chunked_kernel<TT, 128><<<items * heads * 8, 256, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, \
                                                                            state_row, state_slots, item_start, o, heads);          \
     else if (d <= 32)                                                                                                                    \
-      time_scan_kernel<TT, 8><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
+      time_scan_kernel<TT, 2><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
                                                               state_slots, item_start, o, heads, d);                                \
     else if (d <= 64)                                                                                                               \
-      time_scan_kernel<TT, 16><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
+      time_scan_kernel<TT, 4><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
                                                                state_slots, item_start, o, heads, d);                               \
     else if (d <= 128)                                                                                                              \
-      time_scan_kernel<TT, 32><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
+      time_scan_kernel<TT, 8><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
                                                                state_slots, item_start, o, heads, d);                               \
     else                                                                                                                            \
-      time_scan_kernel<TT, 64><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
+      time_scan_kernel<TT, 16><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
                                                                state_slots, item_start, o, heads, d);                               \
     time_finish_kernel<TT><<<fin_blocks, 256, 0, stream>>>(o, (const TT*)gate, norm_w, (TT*)out, out_row, out_col, out_scale, units,  \
                                                            heads, d, eps);                                                          \

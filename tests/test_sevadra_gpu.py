@@ -141,6 +141,8 @@ def one_layer_models() -> dict[str, dict]:
         "attention without convolution and rotation": sh.model(90, 64, 1e-5, 0, [sh.layer(sh.attention(2, 2, 32, 32, 0.2))]),
         "a pair of capped attention and time mixing": sh.model(90, 64, 1e-5, 0, [sh.layer(sh.parallel((4, 1, 16, 16, 0.4, 1.0), (4, 16, 8), 0.5, 1.5))]),
         "time mixing beside a silent attention": sh.model(90, 64, 1e-5, 0, [sh.layer(sh.parallel((1, 1, 16, 16, 0.4, 5.0), (2, 32, 4), 0.0, 1.0))]),
+        "time mixing over one head of 128 and over heads of 32": sh.model(90, 64, 1e-5, 0, [
+            sh.layer(sh.parallel((2, 1, 16, 16, 0.4, 5.0), (1, 128, 8), 0.3, 1.0)), sh.layer(sh.parallel((2, 2, 16, 16, 0.4, 5.0), (3, 32, 5), 0.5, 0.8))]),
         "latent attention": sh.model(90, 64, 1e-5, 0, [sh.layer(sh.latent(3, 16, 8, 24, 40, 0.25, 10000.0))]),
         "latent attention over another layer's latents": sh.model(90, 64, 1e-5, 0, [sh.layer(sh.latent(3, 16, 8, 24, 40, 0.25, 10000.0)),
                                                                                     sh.layer(sh.latent(5, 8, 8, 16, 40, 0.3, 10000.0, kv_from=0))]),
