@@ -130,12 +130,12 @@ class AttentionSpec:
     # left the window and whose block is not yet complete behind it are not seen
     pooled_block: int = 0
     # with q and k normed over the whole projection: > 0, a short causal convolution over time of that many taps on every channel of
-    # q, k and v, directly behind the projections (``y_t = sum_j w[:, j] u_(t - taps + 1 + j)``, zeros before the sequence; weights
+    # q, k and v, directly behind the projections (``y_t = sum_j w[:, j] u_(t - taps + 1 + j)``, nothing but zeros ahead of a sequence's first token; weights
     # ``[channels, taps]`` under the roles ``q_conv k_conv v_conv``); the last ``taps - 1`` projections of a sequence are its state
     conv_taps: int = 0
     # > 0: every scaled score s becomes softcap * tanh(s / softcap) before the softmax
     softcap: float = 0.0
-    # one is added to the softmax's denominator: a sink whose score is 0 and which has no value
+    # the softmax's denominator holds one more term, exp(0), that carries no value (a sink with the logit 0)
     unit_sink: bool = False
 
     @property
@@ -385,7 +385,7 @@ class LayerSpec:
     feed-forward has a norm of its own, of the same x: ``x += residual_scale * (mixer(norm1(x)) + ffn(norm2(x)))``.
     ``arrangement == "hyper_connections"``: as ``pre_norm`` over several residual streams: each part reads and rewrites them by
     its :class:`HyperConnectionSpec` (``mixer_streams``, ``ffn_streams``); ``ffn`` may be None.
-    ``arrangement == "result_norm"``: the norms sit on the sublayers' results, and the sublayers read the stream itself:
+    ``arrangement == "result_norm"``: the norms sit on the sublayers' results, and what a sublayer takes in is the stream as it stands:
     ``x += norm1(mixer(x)); x += norm2(ffn(x))``; ``ffn`` may be None. ``token_input`` (any arrangement that takes it): an input from
     the token itself behind the feed-forward (:class:`TokenInputSpec`).
     The ``*_prefix`` / ``*_name`` strings are the checkpoint names of this layer's tensors.

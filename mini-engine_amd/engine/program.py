@@ -195,7 +195,7 @@ class StepProgram:
         self._stream_rewrite: torch.Tensor | None = None  # how the pending result rewrites the streams (mix, then out)
         self.draws = False
         # the residual stream in the compute dtype as the last norm of a sublayer's result left it (a value that no scope owns), for
-        # blocks whose sublayers read the stream itself
+        # blocks whose sublayers take in the stream as it stands
         self.stream_value: int | None = None
         self.last_prefill_columns = 0  # query columns of the prefill attention's blocks in the last eager step (0: none ran)
         # called parts: their C trampolines (kept alive), the memory and the batch of the step that is running,

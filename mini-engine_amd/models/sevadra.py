@@ -1,7 +1,7 @@
 """The Sevadra decoder: its ``config.json`` keys, and the plan that assembles it from parts.
 
 A Sevadra model is a list of layers whose norms sit on the sublayers' results: ``x += norm1(mixer(x))``, ``x += norm2(ff(x))`` (RMS
-norms; the sublayers read the stream itself; the feed-forward may be absent), and, when the config has ``token_side``, an input
+norms; what a sublayer takes in is the stream as it stands; the feed-forward may be absent), and, when the config has ``token_side``, an input
 from the token itself behind the feed-forward of every layer: with e the layer's ``dim`` elements of the token's row of a table,
 ``y = W_proj (gelu_tanh(W_gate x) * e)`` and ``x += rmsnorm(y) * w``. The head is the embedding table behind the final norm.
 
@@ -12,7 +12,7 @@ Three mixers (``type`` of a layer entry):
                       ``rot.dims`` elements of a head, slow pairs slowed by ``rot.scaling`` (factor, low, high, original).
 ``parallel``          a pair of mixers that read the same input, ``left_scale * left + right_scale * right``. Left: attention
                       without rotation, q and k normed over their whole projection, scores bounded by ``softcap * tanh(s / softcap)``,
-                      one added to the softmax's denominator. Right: linear attention with a decay per token and channel and a
+                      a softmax whose denominator holds one more term, exp(0). Right: linear attention with a decay per token and channel and a
                       bonus for the current token, every projection reading its own blend of the token and the one before.
 ``latent_attention``  attention over one cached latent per token (``kv_rank`` elements) and a turned key part that all heads share
                       (``rot_dim`` elements, pairs of neighbours), a sigmoid gate per head; with ``kv_from: j`` the layer reads
@@ -20,7 +20,7 @@ Three mixers (``type`` of a layer entry):
 
 Two feed-forwards (``mlp.kind``): ``dense``, ``down(relu(up x)^2)``; ``moe``, ``router.experts`` such feed-forwards of ``expert.ff``
 of which a token uses ``router.top``: scores are the softmax over all router outputs, picked by score plus ``correction``, weighted
-by the scores as they are; the last ``router.identity`` outputs are identity experts (the input itself); an optional ``shared``
+by the scores as they are; the last ``router.identity`` outputs are identity experts (they hand the token's input on); an optional ``shared``
 expert runs for every token.
 
 config.json keys: ``architecture``, ``vocab``, ``width``, ``norm`` (``eps``), ``token_side`` (``dim``) or absent, ``layers`` (each ``type``,

@@ -13,7 +13,7 @@ norm of its own for the feed-forward (both norms of the same x)::
 
     x = x + scale * (mixer(norm1(x)) + ffn(norm2(x)))
 
-``result_norm``: the norms sit on the sublayers' results and the sublayers read the stream itself::
+``result_norm``: the norms sit on the sublayers' results and what a sublayer takes in is the stream as it stands::
 
     x = x + norm1(mixer(x));  x = x + norm2(ffn(x))
 

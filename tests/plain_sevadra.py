@@ -2,7 +2,7 @@
 once, no cache and no batching. It shares no code with the package; the tests hold the engine against it.
 
 ``w`` maps tensor names to tensors; ``cfg`` is the dictionary of ``config.json``. A layer is ``x += norm1(mixer(x))``, ``x +=
-norm2(ff(x))`` (the norm on the sublayer's result; the sublayers read the stream itself), then a per-layer token input.
+norm2(ff(x))`` (the norm on the sublayer's result; what a sublayer takes in is the stream as it stands), then a per-layer token input.
 """
 
 from __future__ import annotations
@@ -114,7 +114,7 @@ def attention_mixer(h, w, p: str, m: dict, eps: float):
 
 
 def capped_sink_attention(h, w, p: str, m: dict, eps: float):
-    """The left mixer of a pair: no rotation, scores bounded by ``softcap``, one added to the softmax's denominator."""
+    """The left mixer of a pair: no rotation, scores bounded by ``softcap``, a softmax whose denominator holds one more term, exp(0)."""
     t = h.shape[0]
     heads, kv, d, dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
     q = rms_norm(h @ w[p + ".q"].T, w[p + ".q.norm"], eps).reshape(t, heads, d)
