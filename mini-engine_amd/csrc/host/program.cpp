@@ -178,6 +178,7 @@ bool pooled_takes_matrix_cores(const Op& op, int dtype, long long out_row) {
 
 int groups_of(int64_t v) { return v > 1 ? (int)v : 1; }
 bool act_code_is_ungated(int code) { return code >= 16; }  // csrc/common.h: MeAct
+constexpr int kTimeMixStackedTokens = 32;  // up to here time mixing's five products are one (Run::time_mix)
 float scale_of(float f) { return f == 0.f ? 1.f : f; }
 
 class Run {
@@ -367,6 +368,25 @@ class Run {
   void time_mix(const Op& op) {
     const int heads = (int)op.i[0], d = (int)op.i[1], rank = (int)op.i[2], n = heads * d;
     const long long state_row = op.i[4], prev_at = op.i[5];
+    if (op.p[11] && t_ <= kTimeMixStackedTokens) {
+      // Few tokens (decode steps): the five blends of a token are five rows of ONE product with the five weights stacked. A row meets
+      // all of the stacked weight, of which its own fifth is used: five times the multiply-adds, but the weights are read once and the
+      // step waits for one product, not five (at these sizes a product is the time its weights take to arrive).
+      const long long wide = 4ll * n + rank;
+      char* x5 = (char*)arena_.take((size_t)5 * t_ * h_ * elem_);
+      char* p5 = (char*)arena_.take((size_t)5 * t_ * wide * elem_);
+      void* ws = arena_.take((size_t)me_time_mix_workspace(t_, heads, d));
+      void* rows[5];
+      for (int i = 0; i < 5; ++i) rows[i] = x5 + (size_t)i * h_ * elem_;
+      ok(me_time_shift(bufs_[op.in], (float*)op.p[7], state_row, prev_at, idx(s_.lay.state_slots), idx(s_.lay.item_start), idx(s_.lay.token_item),
+                       idx(s_.lay.positions), (const float*)op.p[0], rows, 5ll * h_, t_, s_.lay.items, h_, dtype_, stream_));
+      product(x5, op.p[11], (int)wide, h_, 0, dtype_, p5, kRolePlain, 5 * t_);
+      auto at = [&](int i) { return p5 + ((size_t)i * wide + (size_t)i * n) * elem_; };  // blend i's row of a token, at its own columns
+      ok(me_time_mix(at(0), at(1), at(2), at(3), at(4), op.p[3], (const float*)op.p[4], (const float*)op.p[5], (const float*)op.p[6],
+                     (float*)op.p[7], state_row, idx(s_.lay.state_slots), idx(s_.lay.item_start), bufs_[op.out], values_[op.out].cols, (int)op.i[3],
+                     op.f[1], t_, s_.lay.items, heads, d, rank, op.f[0], 5 * wide, dtype_, ws, stream_));
+      return;
+    }
     void* mixes[5];
     for (int i = 0; i < 5; ++i) mixes[i] = arena_.take((size_t)t_ * h_ * elem_);
     void* proj[4];
@@ -374,13 +394,13 @@ class Run {
     void* z = arena_.take((size_t)t_ * rank * elem_);
     void* ws = arena_.take((size_t)me_time_mix_workspace(t_, heads, d));
     ok(me_time_shift(bufs_[op.in], (float*)op.p[7], state_row, prev_at, idx(s_.lay.state_slots), idx(s_.lay.item_start), idx(s_.lay.token_item),
-                     idx(s_.lay.positions), (const float*)op.p[0], mixes, t_, s_.lay.items, h_, dtype_, stream_));
+                     idx(s_.lay.positions), (const float*)op.p[0], mixes, h_, t_, s_.lay.items, h_, dtype_, stream_));
     const void* weights[4] = {op.p[1], op.p[8], op.p[9], op.p[10]};  // r, k, v, gate
     for (int i = 0; i < 4; ++i) product(mixes[i], weights[i], n, h_, 0, dtype_, proj[i]);
     product(mixes[4], op.p[2], rank, h_, 0, dtype_, z);
     ok(me_time_mix(proj[0], proj[1], proj[2], proj[3], z, op.p[3], (const float*)op.p[4], (const float*)op.p[5], (const float*)op.p[6],
                    (float*)op.p[7], state_row, idx(s_.lay.state_slots), idx(s_.lay.item_start), bufs_[op.out], values_[op.out].cols, (int)op.i[3],
-                   op.f[1], t_, s_.lay.items, heads, d, rank, op.f[0], dtype_, ws, stream_));
+                   op.f[1], t_, s_.lay.items, heads, d, rank, op.f[0], 0, dtype_, ws, stream_));
   }
 
   void release_parts() {
@@ -1102,7 +1122,7 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
              (size_t)tokens * (4 + 3 * op.i[7] * elem + 2 * op.i[7] * 4) + 6 * pad;
     if (op.kind == kOpTimeMix)
       need = (size_t)tokens * (5 * hidden_ + 4 * op.i[0] * op.i[1] + op.i[2]) * elem + (size_t)me_time_mix_workspace(tokens, (int)op.i[0], (int)op.i[1]) +
-             12 * pad;
+             (size_t)std::min<int64_t>(tokens, kTimeMixStackedTokens) * 5 * (hidden_ + 4 * op.i[0] * op.i[1] + op.i[2]) * elem + 16 * pad;
     if (op.kind == kOpDeltaRule && tokens > items) need = (size_t)me_delta_rule_workspace(tokens, (int)op.i[0], (int)op.i[1]) + pad;
     if (op.kind == kOpPooledAttention) {
       need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;

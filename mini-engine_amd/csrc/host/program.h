@@ -91,7 +91,7 @@ enum OpKind {
   kOpActivate = 24,   // in -> out (the same value or another of its size): act(in) elementwise, i0 the activation's code (MeAct)
   kOpTimeMix = 25,    // linear attention with a decay per token and channel and a bonus for the current token (csrc/time_mix.hip). in: the
                       // sublayer's input [tokens, hidden]; p0 float32 [5, hidden] the blends' mu (r, k, v, gate, decay), p1, p8, p9, p10 W_r, W_k, W_v, W_gate
-                      // [n, hidden] each, p2 W1 [i2, hidden], p3 W2 [n, i2], p4 w0, p5 bonus, p6 weight of the output norm (float32 [n]
+                      // [n, hidden] each (p11, or null: the five weights stacked, [4 n + i2, hidden], for steps of few tokens), p2 W1 [i2, hidden], p3 W2 [n, i2], p4 w0, p5 bonus, p6 weight of the output norm (float32 [n]
                       // each), p7 state rows float32 [slots, i4]: S [heads, d, d], then at i5 the input of the sequence's last token;
                       // i0 heads, i1 d (n = i0 * i1), i2 the decay's inner size, i3 the result's column in out; f0 eps, f1 what multiplies the result
 };

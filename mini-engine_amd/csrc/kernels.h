@@ -222,13 +222,13 @@ int me_conv_norm_rope_scatter(const void* proj, long long row, int c_q, int c_k,
                               void* q_out, void* k_cache, void* v_cache, int num_tokens, int items, int nh, int nkv, int d, int dv, int bs,
                               float eps, int dtype, hipStream_t stream);
 int me_time_shift(const void* h, float* state, long long state_row, long long prev_at, const int* state_slots, const int* item_start,
-                  const int* token_item, const int* positions, const float* mu, void* const* outs, int num_tokens, int items, int width,
-                  int dtype, hipStream_t stream);
+                  const int* token_item, const int* positions, const float* mu, void* const* outs, long long out_stride, int num_tokens, int items,
+                  int width, int dtype, hipStream_t stream);
 long long me_time_mix_workspace(long long tokens, int heads, int d);
 int me_time_mix(const void* r, const void* k, const void* v, const void* gate, const void* z, const void* W2, const float* w0,
                 const float* bonus, const float* norm_w, float* state, long long state_row, const int* state_slots, const int* item_start,
                 void* out, long long out_row, int out_col, float out_scale, int num_tokens, int items, int heads, int d, int rank, float eps,
-                int dtype, void* workspace, hipStream_t stream);
+                long long in_stride, int dtype, void* workspace, hipStream_t stream);
 int me_attention_decode_bf16_placed(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx, const int* block_table,
                                     int table_width, void* out, long long out_row, int out_col, float out_scale, float* part_o,
                                     float* part_ml, int items, int nh, int nkv, int d, int bs, int window, float scale, float softcap,

@@ -24,7 +24,7 @@ __global__ __launch_bounds__(256) void time_shift_kernel(const T* __restrict__ h
                                                          const int* __restrict__ item_start, const int* __restrict__ token_item,
                                                          const int* __restrict__ positions, const float* __restrict__ mu,
                                                          T* __restrict__ o0, T* __restrict__ o1, T* __restrict__ o2, T* __restrict__ o3,
-                                                         T* __restrict__ o4, int width) {
+                                                         T* __restrict__ o4, int width, long long out_stride) {
   const int t = blockIdx.x, item = token_item[t];
   const bool from_state = t == item_start[item];
   const float* prev_row = state + (size_t)state_slots[item] * state_row + prev_at;
@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void time_shift_kernel(const T* __restrict__ h
     const float x = to_float(h[(size_t)t * width + i]);
     const float prev = none ? 0.f : (from_state ? prev_row[i] : to_float(h[(size_t)(t - 1) * width + i]));
     const float dlt = prev - x;
-    const size_t at = (size_t)t * width + i;
+    const size_t at = (size_t)t * out_stride + i;  // (the blends' rows may lie interleaved in one buffer)
     o0[at] = from_float<T>(fmaf(dlt, mu[i], x));
     o1[at] = from_float<T>(fmaf(dlt, mu[width + i], x));
     o2[at] = from_float<T>(fmaf(dlt, mu[2 * width + i], x));
@@ -52,21 +52,22 @@ __global__ __launch_bounds__(256) void time_shift_keep_kernel(const T* __restric
   for (int i = threadIdx.x; i < width; i += blockDim.x) prev_row[i] = to_float(h[(size_t)last * width + i]);
 }
 
-// h [T, width]; mu float32 [5, width] (r, k, v, gate, decay); outs: five [T, width] buffers in the activations' type.
+// h [T, width]; mu float32 [5, width] (r, k, v, gate, decay); outs: five buffers in the activations' type whose rows of `width` elements
+// lie out_stride elements apart (width: five plain [T, width] buffers; 5 * width and bases a row apart: one buffer [T, 5, width]).
 extern "C" int me_time_shift(const void* h, float* state, long long state_row, long long prev_at, const int* state_slots,
                              const int* item_start, const int* token_item, const int* positions, const float* mu, void* const* outs,
-                             int num_tokens, int items, int width, int dtype, hipStream_t stream) {
+                             long long out_stride, int num_tokens, int items, int width, int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (width <= 0 || prev_at < 0 || prev_at + width > state_row) return me_fail("me_time_shift: width=%d at %lld of a row of %lld", width, prev_at, state_row);
   if (dtype == ME_F32) {
     time_shift_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)h, state, state_row, prev_at, state_slots, item_start, token_item,
                                                              positions, mu, (float*)outs[0], (float*)outs[1], (float*)outs[2],
-                                                             (float*)outs[3], (float*)outs[4], width);
+                                                             (float*)outs[3], (float*)outs[4], width, out_stride);
     time_shift_keep_kernel<float><<<items, 256, 0, stream>>>((const float*)h, state, state_row, prev_at, state_slots, item_start, width);
   } else {
     time_shift_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)h, state, state_row, prev_at, state_slots, item_start,
                                                               token_item, positions, mu, (bf16_t*)outs[0], (bf16_t*)outs[1],
-                                                              (bf16_t*)outs[2], (bf16_t*)outs[3], (bf16_t*)outs[4], width);
+                                                              (bf16_t*)outs[2], (bf16_t*)outs[3], (bf16_t*)outs[4], width, out_stride);
     time_shift_keep_kernel<bf16_t><<<items, 256, 0, stream>>>((const bf16_t*)h, state, state_row, prev_at, state_slots, item_start, width);
   }
   return me_check_launch("me_time_shift");
@@ -93,7 +94,8 @@ template <typename T, int RPL>
 __global__ __launch_bounds__(64) void time_scan_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v,
                                                        const float* __restrict__ decay, const float* __restrict__ bonus,
                                                        float* __restrict__ state, long long state_row, const int* __restrict__ state_slots,
-                                                       const int* __restrict__ item_start, float* __restrict__ o, int heads, int d) {
+                                                       const int* __restrict__ item_start, float* __restrict__ o, int heads, int d,
+                                                       long long in_stride) {
   const int groups = (d + 3) / 4;
   const int item = blockIdx.x / (heads * groups), head = (blockIdx.x / groups) % heads, grp = blockIdx.x % groups;
   const int lane = threadIdx.x, rp = lane & 15, c = grp * 4 + (lane >> 4);
@@ -111,15 +113,15 @@ __global__ __launch_bounds__(64) void time_scan_kernel(const T* __restrict__ r, 
     u[a] = there ? bonus[head * d + i] : 0.f;
   }
   for (int t = first; t < end; ++t) {
-    const size_t at = (size_t)t * n + head * d;
-    const float vc = col ? to_float(v[at + c]) : 0.f;
+    const size_t at = (size_t)t * n + head * d, in = (size_t)t * in_stride + head * d;  // (rows of r, k, v may be wider than n)
+    const float vc = col ? to_float(v[in + c]) : 0.f;
     float rr[RPL], kk[RPL], ww[RPL];
 #pragma unroll
     for (int a = 0; a < RPL; ++a) {
       const int i = i0 + a;
       const bool there = a < per && i < d;
-      rr[a] = there ? to_float(r[at + i]) : 0.f;
-      kk[a] = there ? to_float(k[at + i]) : 0.f;
+      rr[a] = there ? to_float(r[in + i]) : 0.f;
+      kk[a] = there ? to_float(k[in + i]) : 0.f;
       ww[a] = there ? decay[at + i] : 0.f;
     }
     float acc = 0.f;
@@ -181,10 +183,10 @@ struct TsVec<float> {
 #define TD_TOKENS 8
 template <typename T>
 __global__ __launch_bounds__(256) void time_decay_kernel(const T* __restrict__ z, const T* __restrict__ W2, const float* __restrict__ w0,
-                                                         float* __restrict__ decay, int num_tokens, int n, int rank) {
+                                                         float* __restrict__ decay, int num_tokens, int n, int rank, long long z_stride) {
   extern __shared__ float th[];  // [TD_TOKENS][rank]
   const int t0 = blockIdx.x * TD_TOKENS, count = min(TD_TOKENS, num_tokens - t0);
-  for (int i = threadIdx.x; i < count * rank; i += blockDim.x) th[i] = tanhf(to_float(z[(size_t)t0 * rank + i]));
+  for (int i = threadIdx.x; i < count * rank; i += blockDim.x) th[i] = tanhf(to_float(z[(size_t)(t0 + i / rank) * z_stride + i % rank]));
   __syncthreads();
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= n) return;
@@ -326,7 +328,7 @@ __global__ __launch_bounds__(256) void time_scan_chunked_kernel(const T* __restr
 template <typename T>
 __global__ __launch_bounds__(256) void time_finish_kernel(const float* __restrict__ o, const T* __restrict__ gate, const float* __restrict__ w,
                                                           T* __restrict__ out, long long out_row, int out_col, float out_scale,
-                                                          long long units, int heads, int d, float eps) {
+                                                          long long units, int heads, int d, float eps, long long in_stride) {
   const long long unit = (long long)blockIdx.x * (blockDim.x / ME_WAVE) + threadIdx.x / ME_WAVE;
   if (unit >= units) return;
   const int lane = threadIdx.x & (ME_WAVE - 1);
@@ -337,20 +339,21 @@ __global__ __launch_bounds__(256) void time_finish_kernel(const float* __restric
   for (int i = lane; i < d; i += ME_WAVE) ss = fmaf(orow[i], orow[i], ss);
   const float rinv = rsqrtf(wave_sum(ss) / (float)d + eps) * out_scale;
   for (int i = lane; i < d; i += ME_WAVE) {
-    const float g = to_float(gate[(size_t)t * n + head * d + i]);
+    const float g = to_float(gate[(size_t)t * in_stride + head * d + i]);
     out[(size_t)t * out_row + out_col + head * d + i] = from_float<T>(orow[i] * rinv * w[head * d + i] * (g / (1.f + expf(-g))));
   }
 }
 
 extern "C" long long me_time_mix_workspace(long long tokens, int heads, int d) { return 2 * tokens * heads * d * 4 + 512; }
 
-// r, k, v, gate [T, heads * d] and z [T, rank] in the activations' type; W2 [heads * d, rank] in the activations' type; w0, bonus,
+// r, k, v, gate (rows of heads * d elements) and z (rows of rank) in the activations' type, their rows in_stride elements apart (0:
+// plain [T, heads * d] and [T, rank] buffers); W2 [heads * d, rank] in the activations' type; w0, bonus,
 // norm_w float32 [heads * d]; state float32 rows of state_row elements whose first heads * d * d are S. out [T, out_row], the
 // result at column out_col. workspace: me_time_mix_workspace bytes.
 extern "C" int me_time_mix(const void* r, const void* k, const void* v, const void* gate, const void* z, const void* W2, const float* w0,
                            const float* bonus, const float* norm_w, float* state, long long state_row, const int* state_slots,
                            const int* item_start, void* out, long long out_row, int out_col, float out_scale, int num_tokens, int items,
-                           int heads, int d, int rank, float eps, int dtype, void* workspace, hipStream_t stream) {
+                           int heads, int d, int rank, float eps, long long in_stride, int dtype, void* workspace, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (heads <= 0 || d <= 0 || d > 256) return me_fail("me_time_mix: %d heads of %d elements (at most 256)", heads, d);
   if (rank <= 0 || rank > TM_MAX_RANK) return me_fail("me_time_mix: a decay of inner size %d (at most %d)", rank, TM_MAX_RANK);
@@ -364,13 +367,14 @@ extern "C" int me_time_mix(const void* r, const void* k, const void* v, const vo
   const unsigned fin_blocks = (unsigned)((units + 3) / 4);
   // steps that bring an item more than a token or two, heads of 32, 64 or 128 elements, rows at multiples of 16 bytes: the kernel that
   // stages chunks of tokens in LDS
-  const bool chunked = num_tokens >= 4 * items && (d == 32 || d == 64 || d == 128) &&
+  const long long rows_apart = in_stride > 0 ? in_stride : n, z_apart = in_stride > 0 ? in_stride : rank;
+  const bool chunked = in_stride <= 0 && num_tokens >= 4 * items && (d == 32 || d == 64 || d == 128) &&
                        ((((uintptr_t)r | (uintptr_t)k | (uintptr_t)v | (uintptr_t)decay)) & 15) == 0;
 #define ME_TM_RUN(TT)                                                                                                               \
   do {                                                                                                                              \
     time_decay_kernel<TT><<<dim3((num_tokens + TD_TOKENS - 1) / TD_TOKENS, (unsigned)((n + 255) / 256)), 256,                       \
                             (size_t)TD_TOKENS * rank * sizeof(float), stream>>>((const TT*)z, (const TT*)W2, w0, decay, num_tokens,  \
-                                                                                (int)n, rank);                                      \
+                                                                                (int)n, rank, z_apart);                             \
     if (chunked && d == 32)                                                                                                         \
       time_scan_chunked_kernel<TT, 32><<<items * heads * 2, 256, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, \
                                                                           state_row, state_slots, item_start, o, heads);           \
@@ -382,18 +386,18 @@ extern "C" int me_time_mix(const void* r, const void* k, const void* v, const vo
                                                                            state_row, state_slots, item_start, o, heads);          \
     else if (d <= 32)                                                                                                                    \
       time_scan_kernel<TT, 2><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
-                                                              state_slots, item_start, o, heads, d);                                \
+                                                              state_slots, item_start, o, heads, d, rows_apart);                                \
     else if (d <= 64)                                                                                                               \
       time_scan_kernel<TT, 4><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
-                                                               state_slots, item_start, o, heads, d);                               \
+                                                               state_slots, item_start, o, heads, d, rows_apart);                               \
     else if (d <= 128)                                                                                                              \
       time_scan_kernel<TT, 8><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
-                                                               state_slots, item_start, o, heads, d);                               \
+                                                               state_slots, item_start, o, heads, d, rows_apart);                               \
     else                                                                                                                            \
       time_scan_kernel<TT, 16><<<scan_blocks, 64, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)v, decay, bonus, state, state_row, \
-                                                               state_slots, item_start, o, heads, d);                               \
+                                                               state_slots, item_start, o, heads, d, rows_apart);                               \
     time_finish_kernel<TT><<<fin_blocks, 256, 0, stream>>>(o, (const TT*)gate, norm_w, (TT*)out, out_row, out_col, out_scale, units,  \
-                                                           heads, d, eps);                                                          \
+                                                           heads, d, eps, rows_apart);                                                          \
   } while (0)
   if (dtype == ME_F32)
     ME_TM_RUN(float);

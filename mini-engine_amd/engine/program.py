@@ -583,7 +583,7 @@ class StepProgram:
 
     def time_mix(self, h: int, out: int, *, out_col: int, mu: torch.Tensor, w_rkvg: tuple, w1: torch.Tensor, w2: torch.Tensor,
                  w0: torch.Tensor, bonus: torch.Tensor, norm_weight: torch.Tensor, state: torch.Tensor, heads: int, head_dim: int,
-                 eps: float, out_scale: float = 1.0) -> None:
+                 eps: float, out_scale: float = 1.0, w_all: torch.Tensor | None = None) -> None:
         """Linear attention with a decay per token and channel and a bonus for the current token, on the value ``h`` ``[tokens, hidden]``
         (the sublayer's input). ``mu`` float32 ``[5, hidden]`` (the blends of r, k, v, gate, decay with the token before); ``w_rkvg`` four weights ``[n,
         hidden]`` (r, k, v, gate), ``w1`` ``[rank, hidden]``, ``w2`` ``[n, rank]`` in the compute dtype (n = heads * head_dim); ``w0``, ``bonus``, ``norm_weight``
@@ -601,9 +601,11 @@ class StepProgram:
         self._want(w2, self.dtype, (n, rank), "the decay's outer weight")
         for t, what in ((w0, "the decay's bias"), (bonus, "the bonus"), (norm_weight, "weight of the output norm")):
             self._want(t, torch.float32, (n,), what)
+        if w_all is not None:  # r, k, v, gate and w1 behind each other: one product serves a step of few tokens
+            self._want(w_all, self.dtype, (4 * n + rank, self.hidden), "the stacked weights of time mixing")
         row = heads * head_dim * head_dim + self.hidden
         self._want(state, torch.float32, (state.shape[0], row), "state")
-        self.op(TIME_MIX, in_=h, out=out, ptrs=[mu, w_rkvg[0], w1, w2, w0, bonus, norm_weight, state, w_rkvg[1], w_rkvg[2], w_rkvg[3]],
+        self.op(TIME_MIX, in_=h, out=out, ptrs=[mu, w_rkvg[0], w1, w2, w0, bonus, norm_weight, state, w_rkvg[1], w_rkvg[2], w_rkvg[3], w_all],
                 ints=[heads, head_dim, rank, out_col, row, heads * head_dim * head_dim], floats=[eps, out_scale])
 
     # ----------------------------------------------------------- several residual streams

@@ -34,7 +34,7 @@ class TimeMix(Mixer):
         names = dict(getattr(s, "names", ()) or ())
         roles = tuple(f"mu_{b}" for b in BLENDS) + ("r", "k", "v", "g", "w1", "w2", "w0", "u", "norm", "o")
         self._n = {r: names.get(r, r) for r in roles}
-        self.w_in = self.w_o = self.mu = self.w_rkvg = self.w1 = self.w2 = self.w0 = self.bonus = self.norm_w = None
+        self.w_in = self.w_o = self.mu = self.w_rkvg = self.w1 = self.w2 = self.w0 = self.bonus = self.norm_w = self.w_all = None
 
     # ---- weights
     def weight_wants(self, prefix: str) -> dict[str, TensorWant]:
@@ -55,6 +55,8 @@ class TimeMix(Mixer):
         self.mu = torch.stack([tensors[f"{prefix}.{n['mu_' + b]}"] for b in BLENDS]).contiguous()
         self.w_rkvg = tuple(tensors[f"{prefix}.{n[r]}"].contiguous() for r in ("r", "k", "v", "g"))
         self.w1 = tensors[f"{prefix}.{n['w1']}"].contiguous()
+        # the five weights behind each other, for steps of few tokens (one product of five rows a token)
+        self.w_all = torch.cat((*self.w_rkvg, self.w1), dim=0).contiguous()
         self.w2 = tensors[f"{prefix}.{n['w2']}"].contiguous()
         self.w_o = tensors[f"{prefix}.{n['o']}"]
         self.w0, self.norm_w = (tensors[f"{prefix}.{n[r]}"] for r in ("w0", "norm"))
@@ -84,7 +86,7 @@ class TimeMix(Mixer):
             raise RuntimeError("time_mix reads the sublayer's input")
         program.time_mix(h, out, out_col=out_col, mu=self.mu, w_rkvg=self.w_rkvg, w1=self.w1, w2=self.w2, w0=self.w0, bonus=self.bonus,
                          norm_weight=self.norm_w, state=cache.state, heads=self.h, head_dim=self.d, eps=float(self.spec.norm_eps),
-                         out_scale=out_scale)
+                         out_scale=out_scale, w_all=self.w_all)
 
     # ---- step
     def forward(self, h, batch, cache=None):
